@@ -74,6 +74,8 @@ class ModelConfig:
     logit_softcap: float = 0.0
     # hyper-connections (models/negunex.py): number of residual streams, 0 = one plain residual
     hyper_streams: int = 0
+    # hashed bigram table added to the embedding (models/zumizen.py): {buckets, mul_prev, mul_cur} or None
+    bigram: Optional[dict] = None
     name: str = "custom"
 
     def __post_init__(self):
@@ -113,12 +115,12 @@ class ModelConfig:
                 d = json.load(f)
         else:
             d = dict(path_or_dict)
-        if d.get("architecture") == "Mekusun":
+        if d.get("architecture") in ("Mekusun", "Zumizen"):
             shapes = {}
             if isinstance(path_or_dict, (str, os.PathLike)):
                 st = os.path.join(os.path.dirname(p), "model.safetensors")
                 shapes = safetensors_shapes(st) if os.path.exists(st) else {}
-            return mekusun_config(d, shapes)
+            return mekusun_config(d, shapes) if d["architecture"] == "Mekusun" else zumizen_config(d, shapes)
         if d.get("architecture") == "Negunex":
             return negunex_config(d)
         names = {f.name for f in dataclasses.fields(cls)}
@@ -202,6 +204,36 @@ def negunex_config(d: dict) -> ModelConfig:
         rms_norm_eps=d["norm"]["eps"], max_position_embeddings=d.get("max_position", 1 << 20),
         bos_token_id=d.get("bos", 0), eos_token_id=d.get("eos", -1), layer_specs=layers,
         hyper_streams=int(d.get("streams") or 0), name=d.get("name", "negunex"))
+
+
+def zumizen_config(d: dict, shapes: Optional[dict] = None) -> ModelConfig:
+    """A Zumizen ``config.json``: ``layers`` lists every layer (``type`` "parallel" or
+    "channel_delta", the ``mixer``'s sizes and constants, ``mlp`` or null), ``embedding`` the scale
+    and the bigram table's hash, ``norm.eps``, ``logit_softcap``, ``vocab``, ``width``. The ranks of
+    the channel form's decay and gate projections are sizes that only the tensors give: they come
+    from ``shapes``, the checkpoint's name -> shape table (or ``decay_rank`` / ``gate_rank``)."""
+    layers = [json.loads(json.dumps(l)) for l in d["layers"]]
+    for i, l in enumerate(layers):
+        if l["type"] not in ("parallel", "channel_delta"):
+            raise ValueError(f"zumizen: layer {i} has the unknown mixer type {l['type']!r}")
+        if l["type"] == "channel_delta" and shapes:
+            for key, name in (("decay_rank", "a1"), ("gate_rank", "g1")):
+                if key not in l["mixer"] and f"l{i}.mix.{name}" in shapes:
+                    l["mixer"][key] = int(shapes[f"l{i}.mix.{name}"][0])
+    moe = [l["mlp"] for l in layers if l.get("mlp") and l["mlp"].get("kind") == "moe"]
+    att = [l["mixer"]["left"] for l in layers if l["type"] == "parallel"]
+    emb = d.get("embedding") or {}
+    return ModelConfig(
+        model_type="zumizen", hidden_size=d["width"], vocab_size=d["vocab"], num_hidden_layers=len(layers),
+        num_attention_heads=att[0]["heads"] if att else 1, num_key_value_heads=att[0]["kv_heads"] if att else 1,
+        head_dim=att[0]["dim"] if att else 1, v_head_dim=att[0]["vdim"] if att else 0, intermediate_size=0,
+        num_local_experts=max([m["router"]["experts"] for m in moe] or [0]),
+        num_experts_per_tok=max([m["router"]["top"] for m in moe] or [0]),
+        moe_intermediate_size=max([m["expert"]["ff"] for m in moe] or [0]),
+        rms_norm_eps=d["norm"]["eps"], max_position_embeddings=d.get("max_position", 1 << 20),
+        bos_token_id=d.get("bos", 0), eos_token_id=d.get("eos", -1), layer_specs=layers,
+        embedding_scale=emb.get("scale", 1.0), bigram=emb.get("bigram"), logit_softcap=d.get("logit_softcap", 0.0),
+        name=d.get("name", "zumizen"))
 
 
 def _llama(name, d, ffn, L, hq, hkv, vocab=128256, **kw):

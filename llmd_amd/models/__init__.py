@@ -40,6 +40,10 @@ def model_class(cfg: ModelConfig):
         from .negunex import NegunexForCausalLM
 
         return NegunexForCausalLM
+    if t == "zumizen":
+        from .zumizen import ZumizenForCausalLM
+
+        return ZumizenForCausalLM
     raise ValueError(f"unsupported model_type {t!r}")
 
 

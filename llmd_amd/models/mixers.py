@@ -13,6 +13,13 @@ constant is an argument, so another stack can reuse them.
   keys, value mixing with an earlier layer and a sigmoid output gate - each one an option.
 * ``GatedMLP`` / ``ScoreMoE`` - gated feed-forwards (act(gate) * up); experts chosen by softmax
   scores plus a selection-only correction, with identity experts.
+* ``GroupedAttention`` options for position-free stacks: weighted query / key norms, a distance bias
+  per head, chunked visibility, a sink in the softmax's denominator, an output bias.
+* ``GatedDeltaMixer``  - gated delta rule behind short convolutions, its decay one per head or one
+  per head and key channel (low-rank), gate SiLU or sigmoid (low-rank).
+* ``ParallelMixer``    - two mixers that read the same input, their results added with two scales.
+* ``SigmoidMoE``       - gated experts chosen by sigmoid scores whose weight scales the expert's input.
+* ``BigramEmbedding``  - token embedding plus a hashed (previous, current) table.
 
 Recurrent state lives in the engine's state pool (engine/state_cache.py): a mixer with
 ``state_shapes()`` gets its per-slot tensors through ``bind_state``; the step's
@@ -229,11 +236,17 @@ class GroupedAttention(torch.nn.Module):
                  ``shared["v_first"]``; later ones use (1 - vmix) v + vmix v_first, which is what they
                  cache
     gate         multiply the concatenated heads by sigmoid(W_g h) before the output projection
+    norm_weight  the unit norms have weights ``q_norm`` / ``k_norm`` [dim], shared by the heads
+    slopes       "pow2": the score of query i and key j loses 2^(-8 (h + 1) / heads) * (i - j)
+    chunk        > 0: query i sees only keys j >= (i // chunk) * chunk (chunks from position 0)
+    sink         one more score of 0 per head in the softmax's denominator, without a value
+    out_bias     the output projection has a bias
     """
     is_latent = False
 
     def __init__(self, d_model, heads, kv_heads, dim, vdim, scale, rot, eps, max_pos, device, dtype, bias=True,
-                 interleaved=True, unit_norm=True, v_mix=False, gate=True):
+                 interleaved=True, unit_norm=True, v_mix=False, gate=True, norm_weight=False, slopes=None, chunk=0,
+                 sink=False, out_bias=False):
         super().__init__()
         if heads % kv_heads:
             raise ValueError(f"{heads} query heads do not divide over {kv_heads} key/value heads")
@@ -247,7 +260,21 @@ class GroupedAttention(torch.nn.Module):
         self.bias = _param((self.nq + self.nk + self.nv,), device, dtype, fill=0.0)
         self.has_bias = bias
         self.vmix = _param((), device, dtype, fill=0.0)
-        self.o = ColumnLinear(heads * vdim, d_model, shard=False, device=device, dtype=dtype)
+        self.o = ColumnLinear(heads * vdim, d_model, bias=bool(out_bias), shard=False, device=device, dtype=dtype)
+        self.norm_weight, self.chunk = bool(norm_weight), int(chunk)
+        if norm_weight:
+            if not unit_norm:
+                raise ValueError("norm weights need the unit norm")
+            self.q_norm = _param((dim,), device, dtype, fill=1.0)
+            self.k_norm = _param((dim,), device, dtype, fill=1.0)
+        if slopes not in (None, "pow2"):
+            raise ValueError(f"unknown distance slopes {slopes!r}")
+        self.slopes = None
+        if slopes == "pow2":
+            self.slopes = torch.tensor([2.0 ** (-8.0 * (h + 1) / heads) for h in range(heads)], dtype=torch.float32,
+                                       device=device)
+        self.sink_logits = torch.zeros(heads, dtype=torch.float32, device=device) if sink else None
+        self.qk_w32 = None
         self.rot_dims = 0
         if rot:
             self.rot_dims = int(rot["dims"])
@@ -263,8 +290,10 @@ class GroupedAttention(torch.nn.Module):
         self.D, self.window, self.sinks = dim + vdim, 0, None
 
     def finalize(self):
-        self.bias32 = self.bias.data.float()
+        self.bias32 = self.bias.data.float() if self.has_bias else None
         self.lam = float(self.vmix.data.float().item())
+        if self.norm_weight:
+            self.qk_w32 = torch.stack([self.q_norm.data.float(), self.k_norm.data.float()]).contiguous()
 
     def kv_spec(self):
         return 1, self.Hkv, self.dim + self.vdim  # (planes, heads, row): [key | value] per kv head
@@ -287,10 +316,11 @@ class GroupedAttention(torch.nn.Module):
                 v_first = shared["v_first"] = torch.empty(T, self.nv, dtype=torch.float32, device=h.device)
         sm.qkv_rope_cache(p, self.bias32, meta.positions, self.cos_sin, self.Hq, self.Hkv, self.dim, self.vdim,
                           self.rot_dims, self.interleaved, self.eps if self.unit_norm else None, v_first, mode,
-                          self.lam, meta.slot_mapping, self.cache, q)
+                          self.lam, meta.slot_mapping, self.cache, q, self.qk_w32)
         n0 = self.nq + self.nk + self.nv
         gate = p[:, n0:n0 + self.Hq * self.vdim] if self.has_gate else None
-        o = sm.grouped_attention(q, self.cache, self.dim, self.vdim, self.scale, meta.seq, gate)
+        o = sm.grouped_attention(q, self.cache, self.dim, self.vdim, self.scale, meta.seq, gate, self.slopes,
+                                 self.chunk, self.sink_logits)
         return self.o(o)
 
 
@@ -330,3 +360,139 @@ class ScoreMoE(torch.nn.Module):
         logits = F.linear(h.float(), self.router32)
         ids, w = sm.moe_route_scores(logits, self.correction32, self.k)
         return sm.moe_gated_ffn(h, ids, w, self.w1, self.w2, self.act)
+
+
+class GatedDeltaMixer(torch.nn.Module):
+    """Gated delta rule. One projection of the layer input gives [q | k | v | beta | decay | gate]:
+    ``kv_heads`` query/key heads of size ``dim`` and ``heads`` value heads of size ``vdim`` (value
+    head h uses q/k head h // (heads / kv_heads)). q, k and v pass a short causal convolution per
+    channel (``taps`` taps, the last one the current token's, no bias) and SiLU; the scan kernel
+    makes q and k unit vectors, q times dim^-1/2, beta = sigmoid, the decay
+    g = exp(-exp(A_log_h) softplus(a + dt_bias)) and runs S <- g S; u = beta (v - S^T k);
+    S <- S + k u^T; o = S^T q, then the head's RMS norm with ``norm`` [vdim] and the gate.
+
+    channel=False  one decay per head (a = W_a h, [heads]); gate silu(W_g h)
+    channel=True   one decay per head and key channel (a = W_a2 (W_a1 h), [heads * dim], rank
+                   ``decay_rank``); gate sigmoid(W_g2 (W_g1 h)), rank ``gate_rank``
+
+    State per sequence: the last taps - 1 inputs of the convolutions and S [heads, dim, vdim] fp32."""
+
+    def __init__(self, d_model, heads, kv_heads, dim, vdim, taps, eps, device, dtype, channel=False, decay_rank=0,
+                 gate_rank=0):
+        super().__init__()
+        if heads % kv_heads:
+            raise ValueError(f"{heads} value heads do not divide over {kv_heads} query/key heads")
+        self.H, self.G, self.dk, self.dv, self.taps, self.eps = heads, kv_heads, dim, vdim, taps, eps
+        self.channel, self.dtype = bool(channel), dtype
+        self.nqk, self.nv = kv_heads * dim, heads * vdim
+        self.C = 2 * self.nqk + self.nv
+        if channel and (decay_rank <= 0 or gate_rank <= 0):
+            raise ValueError("the channel form needs the ranks of its decay and gate projections")
+        self.n_dec = decay_rank if channel else heads
+        self.n_gate = gate_rank if channel else self.nv
+        n = self.C + heads + self.n_dec + self.n_gate
+        self.n_out = -(-n // 8) * 8  # rows of 16-byte multiples
+        self.proj = ColumnLinear(d_model, self.n_out, shard=False, device=device, dtype=dtype)
+        self.conv = _param((self.C, taps), device, dtype, std=0.2)
+        self.register_buffer("conv_b", torch.zeros(self.C, device=device, dtype=dtype), persistent=False)
+        self.A_log = _param((heads,), device, dtype, fill=0.0)
+        self.dt_bias = _param((heads * dim if channel else heads,), device, dtype, fill=0.0)
+        self.norm = _param((vdim,), device, dtype, fill=1.0)
+        if channel:
+            self.a2 = ColumnLinear(decay_rank, heads * dim, shard=False, device=device, dtype=dtype)
+            self.g2 = ColumnLinear(gate_rank, self.nv, shard=False, device=device, dtype=dtype)
+        self.o = ColumnLinear(self.nv, d_model, shard=False, device=device, dtype=dtype)
+        self.A = self.dt_bias32 = None
+        self.conv_state = self.state = None
+
+    def finalize(self):
+        self.A = torch.exp(self.A_log.data.float())
+        self.dt_bias32 = self.dt_bias.data.float()
+
+    def state_shapes(self):
+        return [((max(self.taps - 1, 1), self.C), self.dtype), ((self.H, self.dk, self.dv), torch.float32)]
+
+    def bind_state(self, tensors):
+        self.conv_state, self.state = tensors
+
+    def forward(self, h, meta: AttnMeta):
+        s = meta.seq
+        p = self.proj(h)
+        xc = sm.causal_conv_silu(p, self.C, self.conv, self.conv_b, self.conv_state, s.seq_start, s.seq_slot,
+                                 s.seq_init, s.max_q)
+        c0 = self.C
+        beta = p[:, c0:c0 + self.H]
+        c0 += self.H
+        dec = p[:, c0:c0 + self.n_dec]
+        gate = p[:, c0 + self.n_dec:c0 + self.n_dec + self.n_gate]
+        if self.channel:
+            dec, gate = self.a2(dec), self.g2(gate)
+        y = sm.gated_delta_scan(xc, self.G, self.dk, self.H, self.dv, beta, dec, self.A, self.dt_bias32, gate,
+                                self.channel, self.norm, self.eps, self.state, s)
+        return self.o(y)
+
+
+class ParallelMixer(torch.nn.Module):
+    """Two mixers side by side on the same input; the layer's result is
+    left_scale * left(h) + right_scale * right(h). ``forward`` returns both results and the scales:
+    the sum is taken in fp32 by the kernel that norms it and adds it to the residual."""
+
+    def __init__(self, left, right, left_scale: float, right_scale: float):
+        super().__init__()
+        self.left, self.right = left, right
+        self.left_scale, self.right_scale = float(left_scale), float(right_scale)
+
+    def forward(self, h, meta: AttnMeta):
+        return self.left(h, meta), self.right(h, meta)
+
+
+class SigmoidMoE(torch.nn.Module):
+    """Gated experts W_down (act(W_gate x) * (W_up x)) chosen by score: router logits in fp32, scores
+    = their sigmoids, the ``top`` largest chosen, weights = the chosen scores as they are. The weight
+    multiplies the expert's INPUT: the result is sum_e expert_e(s_e h)."""
+
+    def __init__(self, d_model, ff, experts, top, act, device, dtype):
+        super().__init__()
+        self.E, self.k, self.ff, self.act = experts, top, ff, act
+        self.router = _param((experts, d_model), device, dtype)
+        self.w1 = _param((experts, 2 * ff, d_model), device, dtype)   # [gate rows | up rows]
+        self.w2 = _param((experts, d_model, ff), device, dtype)
+        self.router32 = None
+
+    def finalize(self):
+        self.router32 = self.router.data.float()
+
+    def forward(self, h):
+        logits = F.linear(h.float(), self.router32)
+        ids, w = sm.moe_route(logits, self.k, sigmoid=True)
+        return sm.moe_gated_ffn(h, ids, w, self.w1, self.w2, self.act, scale_input=True)
+
+
+class BigramEmbedding(torch.nn.Module):
+    """x = table[token] * scale + bigram[(previous * mul_prev + token * mul_cur) mod buckets], the
+    table's last row (number ``buckets``) for a sequence's first token; ``bigram`` None: no second
+    table. The previous token of a step's first token is per-sequence state (one int32 per slot)."""
+
+    def __init__(self, vocab, d_model, scale, bigram, device, dtype):
+        super().__init__()
+        from .layers import VocabEmbedding
+
+        self.table = VocabEmbedding(vocab, d_model, device, dtype=dtype)
+        self.scale = float(scale)
+        self.buckets = self.mul_prev = self.mul_cur = 0
+        self.bigram = None
+        if bigram:
+            self.buckets, self.mul_prev, self.mul_cur = (int(bigram[k]) for k in ("buckets", "mul_prev", "mul_cur"))
+            self.bigram = _param((self.buckets + 1, d_model), device, dtype)
+        self.prev = None
+
+    def state_shapes(self):
+        return [((1,), torch.int32)]
+
+    def bind_state(self, tensors):
+        (self.prev,) = tensors
+
+    def forward(self, ids, meta: AttnMeta, x, out_dtype):
+        """Fills the fp32 residual ``x`` [T, d]; returns it in the activation type."""
+        return sm.bigram_embed(ids, self.table.weight, self.scale, self.bigram, self.buckets, self.mul_prev,
+                               self.mul_cur, self.prev, meta.seq, x, out_dtype)

@@ -165,14 +165,16 @@ def xielu(z, ap: float, aq: float):
     return out
 
 
-def moe_route(logits, k: int):
-    """Top-k of fp32 router logits (ties: lower index) and the softmax over the chosen ones."""
+def moe_route(logits, k: int, sigmoid: bool = False):
+    """Top-k of fp32 router logits (ties: lower index) and the softmax over the chosen ones; with
+    ``sigmoid`` the weights are the chosen logits' sigmoids instead, each on its own (the largest
+    sigmoid scores are the largest logits)."""
     if not logits.is_cuda:
-        return ref.moe_route(logits, k)
+        return ref.moe_route(logits, k, sigmoid)
     T = logits.shape[0]
     ids = torch.empty(T, k, dtype=torch.int32, device=logits.device)
     w = torch.empty(T, k, dtype=torch.float32, device=logits.device)
-    native().moe_route(logits, k, ids, w)
+    native().moe_route(logits, k, ids, w, bool(sigmoid))
     return ids, w
 
 
@@ -199,8 +201,8 @@ def moe_ffn(h, ids, w, w1, w2):
     C.moe_group(ids, E, slot_row, tile_e, pair_slot)
     a = torch.empty(max_tiles * MOE_TILE, Fh, dtype=h.dtype, device=dev)
     y = torch.empty(max_tiles * MOE_TILE, d, dtype=h.dtype, device=dev)
-    C.moe_gemm(h, k, slot_row, tile_e, w1, a, 1, n)   # n = rows of the step: picks the tile width
-    C.moe_gemm(a, 0, slot_row, tile_e, w2, y, 0, n)
+    C.moe_gemm(h, k, slot_row, tile_e, w1, a, 1, n, None)   # n = rows of the step: picks the tile width
+    C.moe_gemm(a, 0, slot_row, tile_e, w2, y, 0, n, None)
     out = torch.empty_like(h)
     C.moe_combine(y, pair_slot, w, out, None)
     return out
@@ -236,7 +238,7 @@ def hyper_update_norm(X, y, mix, w_out, next_in=None, next_w=None, eps: float = 
 
 # ---- grouped-query attention with its own key and value sizes
 def qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit_eps, v_first,
-                   v_mode, lam, slots, cache, q_out):
+                   v_mode, lam, slots, cache, q_out, qk_w=None):
     """From a fused projection [q | k | v | ...] of a step's tokens: add ``bias`` (fp32, over q|k|v),
     rotate the first ``rot_dims`` dimensions of every query and key head by the angles of ``cos_sin``
     [max_pos, rot_dims] = [cos | sin] (pairs (2i, 2i+1) when ``interleaved``, (i, i + rot_dims/2)
@@ -244,13 +246,14 @@ def qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, 
     those of an earlier layer (``v_mode`` 1: store this layer's values in ``v_first`` fp32
     [T, Hkv * vdim]; 2: v <- (1 - lam) v + lam v_first), write queries to ``q_out`` [T, Hq, dim] and
     the row [key | value] of every kv head to the paged ``cache`` [blocks, Hkv, bs, dim + vdim] at
-    ``slots`` (-1: no write). All arithmetic fp32."""
+    ``slots`` (-1: no write). ``qk_w`` fp32 [2, dim]: weights of the query and of the key norm (with
+    ``unit_eps``), shared by the heads. ``bias`` may be None. All arithmetic fp32."""
     if not qkv.is_cuda:
         return ref.qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit_eps,
-                                  v_first, v_mode, lam, slots, cache, q_out)
+                                  v_first, v_mode, lam, slots, cache, q_out, qk_w)
     native().qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, bool(interleaved),
                             unit_eps is not None, float(unit_eps or 0.0), v_first, int(v_mode), float(lam), slots, cache,
-                            q_out)
+                            q_out, qk_w)
 
 
 GQA_MFMA = os.environ.get("LLMD_GQA_MFMA", "1") == "1"
@@ -261,11 +264,16 @@ GQA_DECODE_WGS = int(os.environ.get("LLMD_GQA_DECODE_WGS", "2048"))  # workgroup
 GQA_RB2 = os.environ.get("LLMD_GQA_RB2", "0") == "1"
 
 
-def grouped_attention(q, cache, dim, vdim, scale: float, seq, gate=None):
+def grouped_attention(q, cache, dim, vdim, scale: float, seq, gate=None, slopes=None, chunk: int = 0, sinks=None):
     """Causal softmax attention of q [T, Hq, dim] over the paged cache [blocks, Hkv, bs, dim + vdim]
     (query head h reads kv head h // (Hq / Hkv)); row t sees the first seq.row_len[t] keys of its
     sequence. ``gate`` [T, Hq * vdim] (a column view of the fused projection): the result is
     multiplied by sigmoid(gate). Returns [T, Hq * vdim].
+
+    ``slopes`` fp32 [Hq]: the score of query i and key j loses slopes[h] * (i - j).
+    ``chunk`` > 0: query i sees key j only inside its own chunk, j >= (i // chunk) * chunk, chunks
+    counted from the sequence's position 0.
+    ``sinks`` fp32 [Hq]: one more score per head in the softmax's denominator, without a value.
 
     bfloat16 runs on the matrix cores (work item = up to 64 (token, head-of-group) rows of one
     sequence and kv head); float32 and sizes outside the compiled forms on the fp32 FMA kernel."""
@@ -273,28 +281,32 @@ def grouped_attention(q, cache, dim, vdim, scale: float, seq, gate=None):
     Hkv = cache.shape[1]
     out = torch.empty(T, Hq * vdim, dtype=q.dtype, device=q.device)
     if not q.is_cuda:
-        return ref.grouped_attention(q, cache, dim, vdim, seq.tables, seq.row_seq, seq.row_len, scale, gate, out)
+        return ref.grouped_attention(q, cache, dim, vdim, seq.tables, seq.row_seq, seq.row_len, scale, gate, out,
+                                     slopes, chunk, sinks)
     G = Hq // Hkv
+    chunk = int(chunk)
+    # keys a row can see at most: with chunks, its chunk (and the tile that the chunk starts in)
+    span = min(seq.max_len, chunk + 32) if chunk else seq.max_len
     if GQA_MFMA and q.dtype == torch.bfloat16 and G <= 64:
         rb = 2 if GQA_RB2 and seq.max_q * G > 64 else 1
         # workgroup ids run over the kv heads first: ids 256 apart (256 // Hkv items apart) share a CU
         items = seq.attention_items(max(1, 64 * rb // G), balance=max(1, 256 // Hkv) if seq.max_q > 1 else 0)
         nsplit, split, po, pm = 1, 0, None, None
-        if seq.max_q == 1 and seq.max_len > 256:
+        if seq.max_q == 1 and span > 256:
             # decode-only step: key ranges so that items x kv heads x ranges give the chip about
             # eight workgroups per CU (a workgroup walks its tiles one after another)
             n = items.shape[0] * Hkv
-            nsplit = max(1, min(-(-GQA_DECODE_WGS // n), seq.max_len // 128))
-            split = -(-seq.max_len // (nsplit * 32)) * 32
-            nsplit = -(-seq.max_len // split)
+            nsplit = max(1, min(-(-GQA_DECODE_WGS // n), span // 128))
+            split = -(-span // (nsplit * 32)) * 32
+            nsplit = -(-span // split)
             if nsplit > 1:
                 po = torch.empty(n * nsplit * 64 * vdim, dtype=torch.float32, device=q.device)
                 pm = torch.empty(n * nsplit * 128, dtype=torch.float32, device=q.device)
         if native().grouped_attention_mfma(q, cache, dim, vdim, seq.tables, items, seq.row_len, float(scale), gate,
-                                           out, nsplit, split, po, pm, rb):
+                                           out, nsplit, split, po, pm, rb, slopes, chunk, sinks):
             return out
     native().grouped_attention(q, cache, dim, vdim, seq.tables, seq.row_seq, seq.row_len, float(scale), gate,
-                               4 if seq.max_q > 1 else 1, out)
+                               4 if seq.max_q > 1 else 1, out, slopes, chunk, sinks)
     return out
 
 
@@ -322,13 +334,18 @@ def moe_route_scores(logits, correction, k: int):
     return ids, w
 
 
-def moe_gated_ffn(h, ids, w, w1, w2, kind: str = "silu"):
+def moe_gated_ffn(h, ids, w, w1, w2, kind: str = "silu", scale_input: bool = False):
     """sum_j w[t, j] * W2[e] (act(Wg[e] h_t) * (Wu[e] h_t)), e = ids[t, j]; w1 [E, 2F, d] holds
     [gate rows | up rows], w2 [E, d, F]. ids >= E name identity experts: their output is h_t itself.
     Same grouping, tile GEMMs and fp32 combine as ``moe_ffn``; the activation and the product are the
-    first GEMM's epilogue (a workgroup computes matching gate and up columns)."""
+    first GEMM's epilogue (a workgroup computes matching gate and up columns).
+
+    ``scale_input``: the weight multiplies the expert's input instead of its output,
+    sum_j W2[e] (act(Wg[e] (w h_t)) * (Wu[e] (w h_t))): the first GEMM's fp32 sums are scaled by the
+    pair's weight before the activation (both products are linear in the input) and the combine adds
+    the rows as they are. No identity experts in this form."""
     if not h.is_cuda:
-        return ref.moe_gated_ffn(h, ids, w, w1, w2, kind)
+        return ref.moe_gated_ffn(h, ids, w, w1, w2, kind, scale_input)
     C = native()
     T, d = h.shape
     k = ids.shape[1]
@@ -343,10 +360,10 @@ def moe_gated_ffn(h, ids, w, w1, w2, kind: str = "silu"):
     C.moe_group(ids, E, slot_row, tile_e, pair_slot)
     a = torch.empty(max_tiles * MOE_TILE, Fh, dtype=h.dtype, device=dev)
     y = torch.empty(max_tiles * MOE_TILE, d, dtype=h.dtype, device=dev)
-    C.moe_gemm(h, k, slot_row, tile_e, w1, a, 2 + ACT_KINDS[kind], n)
-    C.moe_gemm(a, 0, slot_row, tile_e, w2, y, 0, n)
+    C.moe_gemm(h, k, slot_row, tile_e, w1, a, 2 + ACT_KINDS[kind], n, w if scale_input else None)
+    C.moe_gemm(a, 0, slot_row, tile_e, w2, y, 0, n, None)
     out = torch.empty_like(h)
-    C.moe_combine(y, pair_slot, w, out, h)
+    C.moe_combine(y, pair_slot, None if scale_input else w, out, h)
     return out
 
 
@@ -356,3 +373,56 @@ def softcap_(logits, cap: float):
         return ref.softcap_(logits, cap)
     native().softcap(logits, float(cap))
     return logits
+
+
+# ---- bigram embedding, post-norm residual, gated delta rule
+def bigram_embed(ids, table, scale: float, bigram, buckets: int, mul_prev: int, mul_cur: int, prev_state, seq, x,
+                 out_dtype):
+    """x = table[ids] * scale + bigram[row] (fp32) and its copy in the activation type. The row of a
+    token is (previous token * mul_prev + token * mul_cur) mod buckets, row ``buckets`` for a
+    sequence's first token; the previous token of a run's first token is the sequence's state
+    ``prev_state`` [slots, 1] int32 (read when seq_init is set; the run's last token is written
+    back). ``bigram`` None: the scaled embedding alone."""
+    if not ids.is_cuda:
+        return ref.bigram_embed(ids, table, scale, bigram, buckets, mul_prev, mul_cur, prev_state, seq.seq_start,
+                                seq.seq_slot, seq.seq_init, x, out_dtype)
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    native().bigram_embed(ids, table, float(scale), bigram, int(buckets), int(mul_prev), int(mul_cur), prev_state,
+                          seq.row_seq, seq.seq_start, seq.seq_slot, seq.seq_init, x, out)
+    return out
+
+
+def post_norm_add(y, w_post, x, eps: float, out_dtype, next_w=None, y2=None, a: float = 1.0, b: float = 1.0,
+                  bias=None):
+    """x += rms_norm(a y + b y2 + bias) * w_post on the fp32 residual, in place (plain weights, eps
+    inside the root; ``y2`` and ``bias`` optional). Returns the next reader's input from the same
+    pass: x in the activation type, or rms_norm(x) * next_w when ``next_w`` is given."""
+    if not x.is_cuda:
+        return ref.post_norm_add(y, w_post, x, eps, out_dtype, next_w, y2, a, b, bias)
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    native().post_norm_add(y, y2, float(a), float(b), bias, w_post, x, float(eps), next_w, out)
+    return out
+
+
+def gated_delta_scan(xc, G: int, dk: int, H: int, dv: int, beta_raw, decay_raw, A, dt_bias, gate_raw,
+                     gate_sigmoid: bool, norm_w, eps: float, state, seq):
+    """Gated delta rule over a step's runs. ``xc`` [T, 2 G dk + H dv] = [q | k | v] after the short
+    convolution and SiLU (G query/key heads of size dk, H value heads of size dv, value head h uses
+    q/k head h // (H / G)). Per token and head, all fp32: q and k become unit vectors
+    (x / sqrt(sum x^2 + 1e-6)), q times dk^-1/2; beta = sigmoid(beta_raw [T, H]); the decay is
+    g = exp(-A_h softplus(decay_raw + dt_bias)), one per head (decay_raw [T, H]) or one per head and
+    key channel (decay_raw [T, H dk], acting on the rows of S); then
+
+        S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+
+    and o / rms(o) * norm_w [dv] * gate, gate = silu(gate_raw) or sigmoid(gate_raw) ([T, H dv]).
+    ``state`` [slots, H, dk, dv] fp32 is continued (seq_init) and written back. beta_raw, decay_raw
+    and gate_raw may be column views of one projection. Returns [T, H dv]."""
+    out = torch.empty(xc.shape[0], H * dv, dtype=xc.dtype, device=xc.device)
+    if not xc.is_cuda:
+        return ref.gated_delta_scan(xc, G, dk, H, dv, beta_raw, decay_raw, A, dt_bias, gate_raw, gate_sigmoid, norm_w,
+                                    eps, state, seq.seq_start, seq.seq_slot, seq.seq_init, out)
+    native().gated_delta_scan(xc, int(G), int(dk), int(H), int(dv), beta_raw, decay_raw, A, dt_bias, gate_raw,
+                              bool(gate_sigmoid), norm_w, float(eps), state, seq.seq_start, seq.seq_slot, seq.seq_init,
+                              out)
+    return out

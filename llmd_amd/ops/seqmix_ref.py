@@ -132,9 +132,9 @@ def xielu(z, ap, aq):
     return torch.where(zf > 0, ap * zf * zf + 0.5 * zf, aq * (torch.expm1(zf) - zf) + 0.5 * zf).to(z.dtype)
 
 
-def moe_route(logits, k):
+def moe_route(logits, k, sigmoid=False):
     top, ids = logits.float().topk(k, -1)
-    return ids.int(), torch.softmax(top, -1)
+    return ids.int(), torch.sigmoid(top) if sigmoid else torch.softmax(top, -1)
 
 
 def moe_ffn(h, ids, w, w1, w2):
@@ -173,10 +173,12 @@ def hyper_update_norm(X, y, mix, w_out, next_in, next_w, eps, out_dtype):
 
 
 def qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit_eps, v_first,
-                   v_mode, lam, slots, cache, q_out):
+                   v_mode, lam, slots, cache, q_out, qk_w=None):
     T = qkv.shape[0]
     nq, nk, nv = Hq * dim, Hkv * dim, Hkv * vdim
-    x = qkv[:, :nq + nk + nv].float() + bias.float()
+    x = qkv[:, :nq + nk + nv].float()
+    if bias is not None:
+        x = x + bias.float()
     q, k, v = x[:, :nq].view(T, Hq, dim), x[:, nq:nq + nk].view(T, Hkv, dim), x[:, nq + nk:].view(T, Hkv, vdim)
     if rot_dims:
         half = rot_dims // 2
@@ -196,6 +198,8 @@ def qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, 
     if unit_eps is not None:
         q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + unit_eps)
         k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + unit_eps)
+        if qk_w is not None:
+            q, k = q * qk_w[0].float(), k * qk_w[1].float()
     if v_mode == 1:
         v_first.copy_(v.reshape(T, nv))
     elif v_mode == 2:
@@ -218,20 +222,27 @@ def kv_views(cache, dim, vdim):
     return flat[:, :, :bs * dim].view(nb, Hkv, bs, dim), flat[:, :, bs * dim:].view(nb, Hkv, vdim, bs)
 
 
-def grouped_attention(q, cache, dim, vdim, tables, row_seq, row_len, scale, gate, out):
+def grouped_attention(q, cache, dim, vdim, tables, row_seq, row_len, scale, gate, out, slopes=None, chunk=0,
+                      sinks=None):
     T, Hq, _ = q.shape
     nb, Hkv, bs, _ = cache.shape
     G = Hq // Hkv
     kc, vc = kv_views(cache, dim, vdim)
     for t in range(T):
         n = int(row_len[t])
+        lo = ((n - 1) // chunk) * chunk if chunk else 0       # the first key of the query's chunk
         bt = tables[int(row_seq[t])].long()
-        ar = torch.arange(n)
-        K = kc[bt[ar // bs], :, ar % bs].float()              # [n, Hkv, dim]
-        V = vc[bt[ar // bs], :, :, ar % bs].float()           # [n, Hkv, vdim]
+        ar = torch.arange(lo, n)
+        K = kc[bt[ar // bs], :, ar % bs].float()              # [n - lo, Hkv, dim]
+        V = vc[bt[ar // bs], :, :, ar % bs].float()           # [n - lo, Hkv, vdim]
         qt = q[t].float().view(Hkv, G, dim)
         s = torch.einsum("hgd,nhd->hgn", qt, K) * scale
-        o = torch.einsum("hgn,nhv->hgv", torch.softmax(s, -1), V).reshape(Hq * vdim)
+        if slopes is not None:
+            s = s - slopes.float().view(Hkv, G, 1) * (n - 1 - ar).float()
+        if sinks is not None:                                   # one more score per head, without a value
+            s = torch.cat([s, sinks.float().view(Hkv, G, 1)], -1)
+        p = torch.softmax(s, -1)[..., :n - lo]
+        o = torch.einsum("hgn,nhv->hgv", p, V).reshape(Hq * vdim)
         if gate is not None:
             o = o * torch.sigmoid(gate[t].float())
         out[t] = o.to(out.dtype)
@@ -253,8 +264,18 @@ def moe_route_scores(logits, correction, k):
     return ids.int(), w / (w.sum(-1, keepdim=True) + 1e-20)
 
 
-def moe_gated_ffn(h, ids, w, w1, w2, kind):
+def moe_gated_ffn(h, ids, w, w1, w2, kind, scale_input=False):
     """w1 [E, 2F, d] = [gate | up] rows, w2 [E, d, F]; ids >= E are identity experts."""
+    if scale_input:
+        E, F2, _ = w1.shape
+        out = torch.zeros(h.shape, dtype=torch.float32)
+        hf = h.float()
+        for e in ids.unique().tolist():
+            t, j = (ids == e).nonzero(as_tuple=True)
+            gu = (hf[t] @ w1[e].float().T) * w[t, j, None]
+            a = (_act(gu[:, :F2 // 2], kind) * gu[:, F2 // 2:]).to(h.dtype).float()
+            out.index_add_(0, t, (a @ w2[e].float().T).to(h.dtype).float())
+        return out.to(h.dtype)
     E, F2, _ = w1.shape
     out = torch.zeros(h.shape, dtype=torch.float32)
     hf = h.float()
@@ -267,3 +288,68 @@ def moe_gated_ffn(h, ids, w, w1, w2, kind):
         a = (_act(gu[:, :F2 // 2], kind) * gu[:, F2 // 2:]).to(h.dtype).float()
         out.index_add_(0, t, (a @ w2[e].float().T).to(h.dtype).float() * w[t, j, None])
     return out.to(h.dtype)
+
+
+# ---- bigram embedding, post-norm residual, gated delta rule
+def bigram_embed(ids, table, scale, bigram, buckets, mul_prev, mul_cur, prev_state, seq_start, seq_slot, seq_init,
+                 x, out_dtype):
+    x.copy_(table[ids].float() * scale)
+    if bigram is not None:
+        rows = torch.empty_like(ids)
+        for i in range(seq_slot.numel()):
+            lo, hi, sl = int(seq_start[i]), int(seq_start[i + 1]), int(seq_slot[i])
+            if hi == lo:
+                continue
+            prev = torch.cat([prev_state[sl].view(1).long(), ids[lo:hi - 1]])
+            rows[lo:hi] = (prev * mul_prev + ids[lo:hi] * mul_cur) % buckets
+            if not int(seq_init[i]):
+                rows[lo] = buckets
+            prev_state[sl] = ids[hi - 1]
+        x.add_(bigram[rows].float())
+    return x.to(out_dtype)
+
+
+def _rms(y, eps):
+    return y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + eps)
+
+
+def post_norm_add(y, w_post, x, eps, out_dtype, next_w=None, y2=None, a=1.0, b=1.0, bias=None):
+    v = a * y.float()
+    if y2 is not None:
+        v = v + b * y2.float()
+    if bias is not None:
+        v = v + bias.float()
+    x.add_(_rms(v, eps) * w_post.float())
+    return (x if next_w is None else _rms(x, eps) * next_w.float()).to(out_dtype)
+
+
+def gated_delta_scan(xc, G, dk, H, dv, beta_raw, decay_raw, A, dt_bias, gate_raw, gate_sigmoid, norm_w, eps, state,
+                     seq_start, seq_slot, seq_init, out):
+    T = xc.shape[0]
+    nq = G * dk
+    rep = H // G
+    per_channel = decay_raw.shape[1] == H * dk
+    qa, ka = xc[:, :nq].float().view(T, G, dk), xc[:, nq:2 * nq].float().view(T, G, dk)
+    va = xc[:, 2 * nq:2 * nq + H * dv].float().view(T, H, dv)
+    qa = qa * torch.rsqrt(qa.pow(2).sum(-1, keepdim=True) + 1e-6) * dk ** -0.5
+    ka = ka * torch.rsqrt(ka.pow(2).sum(-1, keepdim=True) + 1e-6)
+    qa, ka = qa.repeat_interleave(rep, 1), ka.repeat_interleave(rep, 1)
+    beta = torch.sigmoid(beta_raw.float())
+    sp = F.softplus(decay_raw.float() + dt_bias.float())
+    dec = torch.exp(-(A.float().view(H, 1) * sp.view(T, H, -1)))       # [T, H, dk or 1]
+    gt = gate_raw.float().view(T, H, dv)
+    gt = torch.sigmoid(gt) if gate_sigmoid else F.silu(gt)
+    for i in range(seq_slot.numel()):
+        lo, hi, sl = int(seq_start[i]), int(seq_start[i + 1]), int(seq_slot[i])
+        S = state[sl].clone() if int(seq_init[i]) else torch.zeros_like(state[sl])
+        for t in range(lo, hi):
+            S = S * dec[t][:, :, None]
+            u = beta[t][:, None] * (va[t] - torch.einsum("hkv,hk->hv", S, ka[t]))
+            S = S + ka[t][:, :, None] * u[:, None]
+            o = torch.einsum("hkv,hk->hv", S, qa[t])
+            o = _rms(o, eps) * norm_w.float() * gt[t]
+            out[t] = o.reshape(H * dv).to(out.dtype)
+        if hi > lo:
+            state[sl] = S
+    del per_channel
+    return out
