@@ -34,16 +34,25 @@ void sm_hyper_update_norm(float*, const void*, int64_t, const float*, const floa
                           void*, int, int, int, int, hipStream_t);
 void sm_gated_act(const void*, int64_t, int, int, void*, int, int, hipStream_t);
 void sm_qkv_rope_cache(const void*, int64_t, const float*, const int64_t*, const float*, int, int, int, int, int, int,
-                       int, float, float*, int, float, const int64_t*, void*, int, void*, int, int, hipStream_t);
+                       int, float, float*, int, float, const int64_t*, void*, int, void*, const float*, int, int,
+                       hipStream_t);
 int sm_grouped_attention(const void*, const void*, const int*, int, int, const int*, const int*, float, int, int, int,
-                         int, int, int, const void*, int64_t, void*, int, hipStream_t);
+                         int, int, int, const void*, int64_t, void*, int, const float*, int, const float*, hipStream_t);
 int sm_grouped_attention_mfma(const void*, const void*, const int*, int, int, const int*, int, const int*, float, int,
-                              int, int, int, const void*, int64_t, void*, int, int, float*, float*, int, hipStream_t);
+                              int, int, int, const void*, int64_t, void*, int, int, float*, float*, int, const float*,
+                              int, const float*, hipStream_t);
 void sm_moe_route_scores(const float*, const float*, int, int, int*, float*, int, hipStream_t);
-void sm_moe_route(const float*, int, int, int*, float*, int, hipStream_t);
+void sm_moe_route(const float*, int, int, int*, float*, int, int, hipStream_t);
 void sm_moe_group(const int*, int, int, int*, int*, int*, int, hipStream_t);
 void sm_moe_gemm(const void*, int64_t, int, const int*, const int*, const void*, int, int, void*, int, int, int, int,
-                 hipStream_t);
+                 const float*, hipStream_t);
+void sm_bigram_embed(const int64_t*, const void*, float, int64_t, const void*, int64_t, int64_t, int64_t, int*,
+                     const int*, const int*, const int*, const int*, int*, float*, void*, int, int, int, hipStream_t);
+void sm_post_norm_add(const void*, int64_t, const void*, int64_t, float, float, const float*, const void*, float*, float,
+                      const void*, void*, int, int, int, hipStream_t);
+int sm_gated_delta_scan(const void*, int64_t, int, int, int, int, const void*, int64_t, const void*, int64_t, int,
+                        const float*, const float*, const void*, int64_t, int, const void*, float, float*, const int*,
+                        const int*, const int*, void*, int, int, hipStream_t);
 void sm_moe_combine(const void*, const int*, const float*, int, int, void*, const void*, int, int, hipStream_t);
 }
 
@@ -366,7 +375,7 @@ void gated_act(Tensor gu, int64_t F, int64_t kind, Tensor out) {
 void qkv_rope_cache(Tensor qkv, std::optional<Tensor> bias, Tensor positions, std::optional<Tensor> cos_sin, int64_t Hq,
                     int64_t Hkv, int64_t dim, int64_t vdim, int64_t rot_dims, bool interleaved, bool unit, double eps,
                     std::optional<Tensor> v_first, int64_t v_mode, double lam, Tensor slots, Tensor cache,
-                    Tensor q_out) {
+                    Tensor q_out, std::optional<Tensor> qk_w) {
   const c10::hip::OptionalHIPGuard g(dev_of(qkv));
   TORCH_CHECK(qkv.is_cuda() && act_ok(qkv) && qkv.dim() == 2 && qkv.stride(1) == 1, "qkv");
   const int64_t T = qkv.size(0), n = (Hq + Hkv) * dim + Hkv * vdim;
@@ -384,6 +393,10 @@ void qkv_rope_cache(Tensor qkv, std::optional<Tensor> bias, Tensor positions, st
     CHECK_F32(*cos_sin);
     TORCH_CHECK(cos_sin->dim() == 2 && cos_sin->size(1) == rot_dims, "cos_sin [max_pos, rot_dims]");
   }
+  if (qk_w) {
+    CHECK_F32(*qk_w);
+    TORCH_CHECK(unit && qk_w->numel() == 2 * dim, "qk_w [2, dim] goes with the unit norm");
+  }
   TORCH_CHECK(v_mode >= 0 && v_mode <= 2, "v_mode");
   if (v_mode) {
     TORCH_CHECK(v_first.has_value(), "v_first");
@@ -398,12 +411,19 @@ void qkv_rope_cache(Tensor qkv, std::optional<Tensor> bias, Tensor positions, st
   sm_qkv_rope_cache(qkv.data_ptr(), qkv.stride(0), bias ? bias->data_ptr<float>() : nullptr,
                     positions.data_ptr<int64_t>(), rot_dims ? cos_sin->data_ptr<float>() : nullptr, Hq, Hkv, dim, vdim,
                     rot_dims, interleaved ? 1 : 0, unit ? 1 : 0, (float)eps, v_mode ? v_first->data_ptr<float>() : nullptr,
-                    v_mode, (float)lam, slots.data_ptr<int64_t>(), cache.data_ptr(), cache.size(2), q_out.data_ptr(), T,
-                    is_f32(qkv), cur());
+                    v_mode, (float)lam, slots.data_ptr<int64_t>(), cache.data_ptr(), cache.size(2), q_out.data_ptr(),
+                    qk_w ? qk_w->data_ptr<float>() : nullptr, T, is_f32(qkv), cur());
 }
 
 void check_gqa(const Tensor& q, const Tensor& cache, int64_t dim, int64_t vdim, const Tensor& tables,
-               const Tensor& row_len, const std::optional<Tensor>& gate, const Tensor& out) {
+               const Tensor& row_len, const std::optional<Tensor>& gate, const Tensor& out,
+               const std::optional<Tensor>& slopes, int64_t chunk, const std::optional<Tensor>& sinks) {
+  TORCH_CHECK(chunk >= 0 && chunk < (1ll << 30), "chunk");
+  for (const auto* v : {&slopes, &sinks})
+    if (*v) {
+      CHECK_F32(**v);
+      TORCH_CHECK((*v)->numel() == q.size(1), "slopes / sinks: fp32 [Hq]");
+    }
   TORCH_CHECK(q.is_cuda() && act_ok(q) && q.dim() == 3 && q.is_contiguous() && q.size(2) == dim, "q [T, Hq, dim]");
   CHECK_ACT(cache, q);
   CHECK_ACT(out, q);
@@ -421,25 +441,27 @@ void check_gqa(const Tensor& q, const Tensor& cache, int64_t dim, int64_t vdim, 
 }
 
 void grouped_attention(Tensor q, Tensor cache, int64_t dim, int64_t vdim, Tensor tables, Tensor row_seq, Tensor row_len,
-                       double scale, std::optional<Tensor> gate, int64_t rows_per_group, Tensor out) {
+                       double scale, std::optional<Tensor> gate, int64_t rows_per_group, Tensor out,
+                       std::optional<Tensor> slopes, int64_t chunk, std::optional<Tensor> sinks) {
   const c10::hip::OptionalHIPGuard g(dev_of(q));
-  check_gqa(q, cache, dim, vdim, tables, row_len, gate, out);
+  check_gqa(q, cache, dim, vdim, tables, row_len, gate, out, slopes, chunk, sinks);
   CHECK_I32(row_seq);
   TORCH_CHECK(row_seq.numel() == q.size(0) && (rows_per_group == 1 || rows_per_group == 4), "row_seq [T]");
   const int rc = sm_grouped_attention(q.data_ptr(), cache.data_ptr(), tables.data_ptr<int>(), tables.size(1),
                                       cache.size(2), row_seq.data_ptr<int>(), row_len.data_ptr<int>(), (float)scale,
                                       q.size(1), cache.size(1), dim, vdim, q.size(0), rows_per_group,
                                       gate ? gate->data_ptr() : nullptr, gate ? gate->stride(0) : 0, out.data_ptr(),
-                                      is_f32(q), cur());
+                                      is_f32(q), slopes ? slopes->data_ptr<float>() : nullptr, chunk,
+                                      sinks ? sinks->data_ptr<float>() : nullptr, cur());
   TORCH_CHECK(rc == 0, "grouped_attention: head sizes too large for the kernel (vdim <= 1024, one key tile in LDS)");
 }
 
 bool grouped_attention_mfma(Tensor q, Tensor cache, int64_t dim, int64_t vdim, Tensor tables, Tensor items,
                             Tensor row_len, double scale, std::optional<Tensor> gate, Tensor out, int64_t nsplit,
                             int64_t split_keys, std::optional<Tensor> part_o, std::optional<Tensor> part_ml,
-                            int64_t rb) {
+                            int64_t rb, std::optional<Tensor> slopes, int64_t chunk, std::optional<Tensor> sinks) {
   const c10::hip::OptionalHIPGuard g(dev_of(q));
-  check_gqa(q, cache, dim, vdim, tables, row_len, gate, out);
+  check_gqa(q, cache, dim, vdim, tables, row_len, gate, out, slopes, chunk, sinks);
   TORCH_CHECK(q.scalar_type() == torch::kBFloat16, "bf16 only");
   CHECK_I32(items);
   TORCH_CHECK(items.dim() == 2 && items.size(1) == 3, "items [n, 3]");
@@ -459,7 +481,8 @@ bool grouped_attention_mfma(Tensor q, Tensor cache, int64_t dim, int64_t vdim, T
                                            cache.size(2), items.data_ptr<int>(), n, row_len.data_ptr<int>(),
                                            (float)scale, q.size(1), Hkv, dim, vdim, gate ? gate->data_ptr() : nullptr,
                                            gate ? gate->stride(0) : 0, out.data_ptr(), nsplit, split_keys, po, pm,
-                                           rb, cur());
+                                           rb, slopes ? slopes->data_ptr<float>() : nullptr, chunk,
+                                           sinks ? sinks->data_ptr<float>() : nullptr, cur());
   return rc == 0;
 }
 
@@ -476,7 +499,7 @@ void moe_route_scores(Tensor logits, Tensor correction, int64_t k, Tensor ids, T
                       w.data_ptr<float>(), T, cur());
 }
 
-void moe_route(Tensor logits, int64_t k, Tensor ids, Tensor w) {
+void moe_route(Tensor logits, int64_t k, Tensor ids, Tensor w, bool sigmoid) {
   const c10::hip::OptionalHIPGuard g(dev_of(logits));
   CHECK_F32(logits);
   CHECK_I32(ids);
@@ -484,7 +507,7 @@ void moe_route(Tensor logits, int64_t k, Tensor ids, Tensor w) {
   const int T = logits.size(0), E = logits.size(1);
   TORCH_CHECK(logits.dim() == 2 && k >= 1 && k <= E && ids.numel() == (int64_t)T * k && w.numel() == (int64_t)T * k,
               "router shapes");
-  sm_moe_route(logits.data_ptr<float>(), E, k, ids.data_ptr<int>(), w.data_ptr<float>(), T, cur());
+  sm_moe_route(logits.data_ptr<float>(), E, k, ids.data_ptr<int>(), w.data_ptr<float>(), T, sigmoid ? 1 : 0, cur());
 }
 
 void moe_group(Tensor ids, int64_t E, Tensor slot_row, Tensor tile_e, Tensor pair_slot) {
@@ -500,7 +523,8 @@ void moe_group(Tensor ids, int64_t E, Tensor slot_row, Tensor tile_e, Tensor pai
                mt, cur());
 }
 
-void moe_gemm(Tensor A, int64_t kdiv, Tensor slot_row, Tensor tile_e, Tensor W, Tensor C, int64_t act, int64_t rows) {
+void moe_gemm(Tensor A, int64_t kdiv, Tensor slot_row, Tensor tile_e, Tensor W, Tensor C, int64_t act, int64_t rows,
+              std::optional<Tensor> row_w) {
   const c10::hip::OptionalHIPGuard g(dev_of(A));
   TORCH_CHECK(A.is_cuda() && act_ok(A) && A.dim() == 2 && A.stride(1) == 1, "A");
   CHECK_ACT(W, A);
@@ -514,26 +538,129 @@ void moe_gemm(Tensor A, int64_t kdiv, Tensor slot_row, Tensor tile_e, Tensor W, 
   TORCH_CHECK(slot_row.numel() == mt * 64 && C.is_contiguous() && C.dim() == 2 && C.size(0) == mt * 64 &&
                   C.size(1) == N, "C [tiles * 64, N]");
   TORCH_CHECK(kdiv > 0 || A.size(0) == mt * 64, "A rows are the tile slots");
+  if (row_w) {  // indexed by the pair numbers in slot_row: one weight per (token, choice)
+    CHECK_F32(*row_w);
+    TORCH_CHECK(act >= 2 && kdiv > 0 && row_w->numel() == A.size(0) * kdiv, "row_w [T, k] with a gated epilogue");
+  }
   sm_moe_gemm(A.data_ptr(), A.stride(0), kdiv, slot_row.data_ptr<int>(), tile_e.data_ptr<int>(), W.data_ptr(),
-              N, W.size(2), C.data_ptr(), mt, rows, (int)act, is_f32(A), cur());
+              N, W.size(2), C.data_ptr(), mt, rows, (int)act, is_f32(A), row_w ? row_w->data_ptr<float>() : nullptr,
+              cur());
 }
 
-void moe_combine(Tensor y, Tensor pair_slot, Tensor w, Tensor out, std::optional<Tensor> h) {
+void moe_combine(Tensor y, Tensor pair_slot, std::optional<Tensor> w, Tensor out, std::optional<Tensor> h) {
   const c10::hip::OptionalHIPGuard g(dev_of(y));
   TORCH_CHECK(y.is_cuda() && act_ok(y) && y.dim() == 2 && y.is_contiguous(), "y");
   CHECK_I32(pair_slot);
-  CHECK_F32(w);
   CHECK_ACT(out, y);
+  TORCH_CHECK(out.dim() == 2, "out [T, d]");
+  if (out.size(0) == 0) return;
   const int T = out.size(0), d = out.size(1);
-  TORCH_CHECK(out.dim() == 2 && out.is_contiguous() && y.size(1) == d && w.dim() == 2 && w.size(0) == T &&
-                  pair_slot.numel() == w.numel(), "combine shapes");
+  TORCH_CHECK(out.is_contiguous() && y.size(1) == d && pair_slot.numel() % T == 0 && pair_slot.numel() >= T,
+              "combine shapes");
+  const int k = pair_slot.numel() / T;
+  if (w) {  // without weights the rows are added as they are
+    CHECK_F32(*w);
+    TORCH_CHECK(w->dim() == 2 && w->size(0) == T && pair_slot.numel() == w->numel(), "w [T, k]");
+  }
   // h: the tokens' inputs, read for pairs marked -1 (identity experts); without it no pair may be -1
   if (h) {
     CHECK_ACT(*h, y);
     TORCH_CHECK(h->dim() == 2 && h->is_contiguous() && h->size(0) == T && h->size(1) == d, "h [T, d]");
   }
-  sm_moe_combine(y.data_ptr(), pair_slot.data_ptr<int>(), w.data_ptr<float>(), w.size(1), d, out.data_ptr(),
+  sm_moe_combine(y.data_ptr(), pair_slot.data_ptr<int>(), w ? w->data_ptr<float>() : nullptr, k, d, out.data_ptr(),
                  h ? h->data_ptr() : y.data_ptr(), T, is_f32(y), cur());
+}
+
+void bigram_embed(Tensor ids, Tensor table, double scale, std::optional<Tensor> bigram, int64_t buckets,
+                  int64_t mul_prev, int64_t mul_cur, Tensor prev_state, Tensor row_seq, Tensor seq_start,
+                  Tensor seq_slot, Tensor seq_init, Tensor x, Tensor out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(ids));
+  TORCH_CHECK(ids.is_cuda() && ids.scalar_type() == torch::kInt64 && ids.is_contiguous(), "ids: int64");
+  TORCH_CHECK(table.is_cuda() && act_ok(table) && table.dim() == 2 && table.is_contiguous(), "table");
+  const int T = ids.numel(), d = table.size(1);
+  CHECK_F32(x);
+  CHECK_ACT(out, table);
+  TORCH_CHECK(x.dim() == 2 && x.size(0) == T && x.size(1) == d && out.is_contiguous() && out.sizes() == x.sizes(),
+              "x, out [T, d]");
+  CHECK_I32(prev_state);
+  CHECK_I32(row_seq);
+  check_seq(seq_start, seq_slot, seq_init, prev_state.numel());
+  TORCH_CHECK(row_seq.numel() == T, "row_seq [T]");
+  Tensor rows;
+  if (bigram) {
+    CHECK_ACT(*bigram, table);
+    TORCH_CHECK(buckets >= 1 && bigram->dim() == 2 && bigram->is_contiguous() && bigram->size(0) == buckets + 1 &&
+                    bigram->size(1) == d, "bigram [buckets + 1, d]");
+    rows = torch::empty({T}, torch::dtype(torch::kInt32).device(ids.device()));
+  }
+  sm_bigram_embed(ids.data_ptr<int64_t>(), table.data_ptr(), (float)scale, table.size(0),
+                  bigram ? bigram->data_ptr() : nullptr, buckets, mul_prev, mul_cur, prev_state.data_ptr<int>(),
+                  row_seq.data_ptr<int>(), seq_start.data_ptr<int>(), seq_slot.data_ptr<int>(),
+                  seq_init.data_ptr<int>(), bigram ? rows.data_ptr<int>() : nullptr, x.data_ptr<float>(),
+                  out.data_ptr(), T, d, is_f32(table), cur());
+}
+
+void post_norm_add(Tensor y, std::optional<Tensor> y2, double a, double b, std::optional<Tensor> bias, Tensor w_post,
+                   Tensor x, double eps, std::optional<Tensor> next_w, Tensor out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(y));
+  TORCH_CHECK(y.is_cuda() && act_ok(y) && y.dim() == 2 && y.stride(1) == 1, "y");
+  const int T = y.size(0), d = y.size(1);
+  CHECK_F32(x);
+  CHECK_ACT(w_post, y);
+  CHECK_ACT(out, y);
+  TORCH_CHECK(x.dim() == 2 && x.size(0) == T && x.size(1) == d && d <= 65536 && w_post.is_contiguous() &&
+                  w_post.numel() == d && out.is_contiguous() && out.sizes() == x.sizes(), "x, out [T, d]; w [d]");
+  if (y2) {
+    CHECK_ACT(*y2, y);
+    TORCH_CHECK(y2->dim() == 2 && y2->stride(1) == 1 && y2->size(0) == T && y2->size(1) == d, "y2 [T, d]");
+  }
+  if (bias) {
+    CHECK_F32(*bias);
+    TORCH_CHECK(bias->numel() == d, "bias [d]");
+  }
+  if (next_w) {
+    CHECK_ACT(*next_w, y);
+    TORCH_CHECK(next_w->is_contiguous() && next_w->numel() == d, "next_w [d]");
+  }
+  sm_post_norm_add(y.data_ptr(), y.stride(0), y2 ? y2->data_ptr() : nullptr, y2 ? y2->stride(0) : 0, (float)a,
+                   (float)b, bias ? bias->data_ptr<float>() : nullptr, w_post.data_ptr(), x.data_ptr<float>(),
+                   (float)eps, next_w ? next_w->data_ptr() : nullptr, out.data_ptr(), T, d, is_f32(y), cur());
+}
+
+void gated_delta_scan(Tensor xc, int64_t G, int64_t dk, int64_t H, int64_t dv, Tensor beta_raw, Tensor decay_raw,
+                      Tensor A, Tensor dt_bias, Tensor gate_raw, bool gate_sigmoid, Tensor norm_w, double eps,
+                      Tensor state, Tensor seq_start, Tensor seq_slot, Tensor seq_init, Tensor out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(xc));
+  TORCH_CHECK(G >= 1 && H >= 1 && H % G == 0 && dk >= 1 && dv >= 1, "head counts and sizes");
+  TORCH_CHECK(xc.is_cuda() && act_ok(xc) && xc.dim() == 2 && xc.stride(1) == 1 && xc.size(1) >= 2 * G * dk + H * dv,
+              "xc [T, q | k | v]");
+  const int64_t T = xc.size(0);
+  CHECK_ACT(beta_raw, xc);
+  CHECK_ACT(decay_raw, xc);
+  CHECK_ACT(gate_raw, xc);
+  CHECK_ACT(norm_w, xc);
+  CHECK_ACT(out, xc);
+  CHECK_F32(A);
+  CHECK_F32(dt_bias);
+  CHECK_F32(state);
+  for (const Tensor* t : {&beta_raw, &decay_raw, &gate_raw})
+    TORCH_CHECK(t->dim() == 2 && t->size(0) == T && t->stride(1) == 1, "beta / decay / gate: [T, n] rows");
+  const bool per_channel = decay_raw.size(1) == H * dk && dk > 1;
+  TORCH_CHECK(beta_raw.size(1) == H && gate_raw.size(1) == H * dv && (per_channel || decay_raw.size(1) == H),
+              "beta [T, H], decay [T, H] or [T, H dk], gate [T, H dv]");
+  TORCH_CHECK(A.numel() == H && dt_bias.numel() == decay_raw.size(1) && norm_w.is_contiguous() && norm_w.numel() == dv,
+              "A [H], dt_bias like the decay, norm_w [dv]");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == dk && state.size(3) == dv,
+              "state [slots, H, dk, dv]");
+  check_seq(seq_start, seq_slot, seq_init, state.size(0));
+  TORCH_CHECK(out.is_contiguous() && out.dim() == 2 && out.size(0) == T && out.size(1) == H * dv, "out [T, H dv]");
+  const int rc = sm_gated_delta_scan(
+      xc.data_ptr(), xc.stride(0), G, dk, H, dv, beta_raw.data_ptr(), beta_raw.stride(0), decay_raw.data_ptr(),
+      decay_raw.stride(0), per_channel ? 1 : 0, A.data_ptr<float>(), dt_bias.data_ptr<float>(), gate_raw.data_ptr(),
+      gate_raw.stride(0), gate_sigmoid ? 1 : 0, norm_w.data_ptr(), (float)eps, state.data_ptr<float>(),
+      seq_start.data_ptr<int>(), seq_slot.data_ptr<int>(), seq_init.data_ptr<int>(), out.data_ptr(), seq_slot.numel(),
+      is_f32(xc), cur());
+  TORCH_CHECK(rc == 0, "gated_delta_scan: head sizes above 256");
 }
 
 }  // namespace
@@ -563,4 +690,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("moe_group", &moe_group);
   m.def("moe_gemm", &moe_gemm);
   m.def("moe_combine", &moe_combine);
+  m.def("bigram_embed", &bigram_embed);
+  m.def("post_norm_add", &post_norm_add);
+  m.def("gated_delta_scan", &gated_delta_scan);
 }

@@ -1,6 +1,7 @@
 // Row kernels of per-layer stacks: embedding with scale, zero-centred RMS norms on the fp32
 // residual, post-norm + layer scale + residual add (+ the next pre-norm in the same pass),
-// the depth average (+ the norm that follows it), xIELU and the logit soft cap.
+// the depth average (+ the norm that follows it), xIELU and the logit soft cap; the embedding with
+// a hashed bigram table and the plain post-norm residual add of stacks that norm only outputs.
 // One workgroup of 256 threads per token row; the fp32 residual is read and written once.
 #include "seqmix_common.h"
 
@@ -101,9 +102,128 @@ __global__ __launch_bounds__(NT) void softcap_kernel(float* __restrict__ x, floa
   if (i < n) x[i] = cap * tanhf(x[i] / cap);
 }
 
+// Row of the bigram table for every token: (previous * mul_prev + token * mul_cur) mod buckets, row
+// ``buckets`` for a sequence's first token. The previous token of a run's first token is the
+// sequence's state; this kernel only reads it (the embedding kernel that follows writes it).
+__global__ __launch_bounds__(NT) void bigram_rows_kernel(const int64_t* __restrict__ ids, int T, int64_t buckets,
+                                                        int64_t mul_prev, int64_t mul_cur,
+                                                        const int* __restrict__ prev_state,
+                                                        const int* __restrict__ row_seq,
+                                                        const int* __restrict__ seq_start,
+                                                        const int* __restrict__ seq_slot,
+                                                        const int* __restrict__ seq_init, int* __restrict__ rows) {
+  const int t = blockIdx.x * NT + threadIdx.x;
+  if (t >= T) return;
+  const int s = row_seq[t];
+  int64_t prev;
+  if (t > seq_start[s]) prev = ids[t - 1];
+  else if (seq_init[s]) prev = prev_state[seq_slot[s]];
+  else {
+    rows[t] = (int)buckets;
+    return;
+  }
+  int64_t r = (prev * mul_prev + ids[t] * mul_cur) % buckets;
+  if (r < 0) r += buckets;
+  rows[t] = (int)r;
+}
+
+// x = table[id] * scale + bigram[row] (fp32) and its copy in the activation type; the workgroup of a
+// run's last token writes the token into the sequence's state.
+template <typename T>
+__global__ __launch_bounds__(NT) void bigram_embed_kernel(const int64_t* __restrict__ ids, const T* __restrict__ table,
+                                                         float scale, int64_t V, const T* __restrict__ bigram,
+                                                         const int* __restrict__ rows, int* __restrict__ prev_state,
+                                                         const int* __restrict__ row_seq,
+                                                         const int* __restrict__ seq_start,
+                                                         const int* __restrict__ seq_slot, float* __restrict__ x,
+                                                         T* __restrict__ out, int d) {
+  const int64_t row = blockIdx.x;
+  const int64_t id = min(max(ids[row], (int64_t)0), V - 1);  // a bad id must not read outside the table
+  const T* src = table + id * (int64_t)d;
+  const T* big = bigram ? bigram + (int64_t)rows[row] * d : nullptr;
+  for (int c = threadIdx.x; c < d; c += NT) {
+    float v = ld(src + c) * scale;
+    if (big) v += ld(big + c);
+    x[row * d + c] = v;
+    st(out + row * d + c, v);
+  }
+  if (threadIdx.x == 0 && prev_state != nullptr) {
+    const int s = row_seq[row];
+    if (row + 1 == seq_start[s + 1]) prev_state[seq_slot[s]] = (int)ids[row];
+  }
+}
+
+// x += rms_norm(a y + b y2 + bias) * wp;  out = x (activation type) or rms_norm(x) * wn
+template <typename T>
+__global__ __launch_bounds__(NT) void post_norm_add_kernel(const T* __restrict__ y, int64_t y_stride,
+                                                          const T* __restrict__ y2, int64_t y2_stride, float a,
+                                                          float b, const float* __restrict__ bias,
+                                                          const T* __restrict__ wp, float* __restrict__ x, float eps,
+                                                          const T* __restrict__ wn, T* __restrict__ out, int d) {
+  __shared__ float red[NT / 64];
+  const int64_t row = blockIdx.x;
+  const T* yr = y + row * y_stride;
+  const T* y2r = y2 ? y2 + row * y2_stride : nullptr;
+  float* xr = x + row * d;
+  auto val = [&](int c) {
+    float v = a * ld(yr + c);
+    if (y2r) v += b * ld(y2r + c);
+    if (bias) v += bias[c];
+    return v;
+  };
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < d; c += NT) {
+    const float v = val(c);
+    ss += v * v;
+  }
+  ss = block_sum<NT>(ss, red);
+  const float inv = 1.f / sqrtf(ss / (float)d + eps);
+  float s2 = 0.f;
+  for (int c = threadIdx.x; c < d; c += NT) {
+    const float v = xr[c] + val(c) * inv * ld(wp + c);
+    xr[c] = v;
+    s2 += v * v;
+    if (wn == nullptr) st(out + row * d + c, v);
+  }
+  if (wn == nullptr) return;
+  s2 = block_sum<NT>(s2, red);
+  const float inv2 = 1.f / sqrtf(s2 / (float)d + eps);
+  for (int c = threadIdx.x; c < d; c += NT) st(out + row * d + c, xr[c] * inv2 * ld(wn + c));
+}
+
 }  // namespace
 
 extern "C" {
+
+void sm_bigram_embed(const int64_t* ids, const void* table, float scale, int64_t V, const void* bigram,
+                     int64_t buckets, int64_t mul_prev, int64_t mul_cur, int* prev_state, const int* row_seq,
+                     const int* seq_start, const int* seq_slot, const int* seq_init, int* rows, float* x, void* out,
+                     int T, int d, int f32, hipStream_t stream) {
+  if (T == 0) return;
+  if (bigram != nullptr)
+    hipLaunchKernelGGL(bigram_rows_kernel, dim3((T + NT - 1) / NT), dim3(NT), 0, stream, ids, T, buckets, mul_prev,
+                       mul_cur, prev_state, row_seq, seq_start, seq_slot, seq_init, rows);
+  if (f32)
+    hipLaunchKernelGGL((bigram_embed_kernel<float>), dim3(T), dim3(NT), 0, stream, ids, (const float*)table, scale, V,
+                       (const float*)bigram, rows, prev_state, row_seq, seq_start, seq_slot, x, (float*)out, d);
+  else
+    hipLaunchKernelGGL((bigram_embed_kernel<bf16_t>), dim3(T), dim3(NT), 0, stream, ids, (const bf16_t*)table, scale, V,
+                       (const bf16_t*)bigram, rows, prev_state, row_seq, seq_start, seq_slot, x, (bf16_t*)out, d);
+}
+
+void sm_post_norm_add(const void* y, int64_t y_stride, const void* y2, int64_t y2_stride, float a, float b,
+                      const float* bias, const void* wp, float* x, float eps, const void* wn, void* out, int T, int d,
+                      int f32, hipStream_t stream) {
+  if (T == 0) return;
+  if (f32)
+    hipLaunchKernelGGL((post_norm_add_kernel<float>), dim3(T), dim3(NT), 0, stream, (const float*)y, y_stride,
+                       (const float*)y2, y2_stride, a, b, bias, (const float*)wp, x, eps, (const float*)wn,
+                       (float*)out, d);
+  else
+    hipLaunchKernelGGL((post_norm_add_kernel<bf16_t>), dim3(T), dim3(NT), 0, stream, (const bf16_t*)y, y_stride,
+                       (const bf16_t*)y2, y2_stride, a, b, bias, (const bf16_t*)wp, x, eps, (const bf16_t*)wn,
+                       (bf16_t*)out, d);
+}
 
 void sm_embed_scale(const int64_t* ids, const void* table, float scale, float* o0, float* o1, int T, int d,
                     int64_t V, int f32, hipStream_t stream) {

@@ -20,6 +20,11 @@
 //   joins them.
 // Both forms multiply the result by sigmoid(gate) when a gate is given. A row's result depends
 // only on its own keys and the fixed tile sizes.
+// Score options of both forms (each may be off): slopes [Hq] - the score of query i and key j loses
+// slopes[h] (i - j); chunk - query i sees only keys j >= (i / chunk) chunk; sinks [Hq] - one more
+// score per head that enters the softmax's denominator and has no value (the running maximum and
+// sum start from it instead of from nothing). Key tiles start at multiples of the tile size from
+// position 0, so a row's tiles do not depend on what else the step holds.
 #include "seqmix_common.h"
 #include <algorithm>
 
@@ -35,7 +40,7 @@ __global__ __launch_bounds__(NT) void qkv_rope_cache_kernel(
     const T* __restrict__ qkv, int64_t stride, const float* __restrict__ bias, const int64_t* __restrict__ positions,
     const float* __restrict__ cos_sin, int Hq, int Hkv, int dim, int vdim, int rot_dims, int interleaved, int unit,
     float eps, float* __restrict__ v_first, int v_mode, float lam, const int64_t* __restrict__ slots,
-    T* __restrict__ cache, int bs, T* __restrict__ q_out) {
+    T* __restrict__ cache, int bs, T* __restrict__ q_out, const float* __restrict__ qk_w) {
   const int64_t t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int half = rot_dims >> 1;
@@ -84,10 +89,11 @@ __global__ __launch_bounds__(NT) void qkv_rope_cache_kernel(
     if (is_q) dst = q_out + (t * Hq + hd) * dim;
     else if (slot >= 0) dst = cache + (blk * Hkv + (hd - Hq)) * bs * Dr + off * dim;
     if (dst == nullptr) continue;
+    const float* nw = qk_w ? qk_w + (is_q ? 0 : dim) : nullptr;  // the norm's weight, shared by the heads
 #pragma unroll
     for (int i = 0; i < MAXE; ++i) {
       const int e = lane + 64 * i;
-      if (e < dim) st(dst + e, r[i] * inv);
+      if (e < dim) st(dst + e, r[i] * inv * (nw ? nw[e] : 1.f));
     }
   }
   const int nv = Hkv * vdim, vcol0 = (Hq + Hkv) * dim;
@@ -134,7 +140,8 @@ __global__ __launch_bounds__(NT) void qkv_rope_cache_vec_kernel(
     const bf16_t* __restrict__ qkv, int64_t stride, const float* __restrict__ bias,
     const int64_t* __restrict__ positions, const float* __restrict__ cos_sin, int Hq, int Hkv, int dim, int vdim,
     int rot_dims, int interleaved, int unit, float eps, float* __restrict__ v_first, int v_mode, float lam,
-    const int64_t* __restrict__ slots, bf16_t* __restrict__ cache, int bs, bf16_t* __restrict__ q_out) {
+    const int64_t* __restrict__ slots, bf16_t* __restrict__ cache, int bs, bf16_t* __restrict__ q_out,
+    const float* __restrict__ qk_w) {
   const int64_t t = blockIdx.x;
   const int half = rot_dims >> 1;
   const float* cs = rot_dims ? cos_sin + positions[t] * rot_dims : nullptr;  // [cos(half) | sin(half)]
@@ -186,6 +193,11 @@ __global__ __launch_bounds__(NT) void qkv_rope_cache_vec_kernel(
       inv = 1.f / sqrtf(ss / (float)dim + eps);
     }
     if (!on) continue;
+    if (qk_w) {
+      const float* nw = qk_w + (hd < Hq ? 0 : dim) + c * 8;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] *= nw[i];
+    }
     if (hd < Hq) st8(q_out + (t * Hq + hd) * dim + c * 8, x, inv);
     else if (slot >= 0) st8(cache + (blk * Hkv + (hd - Hq)) * bs * Dr + off * dim + c * 8, x, inv);
   }
@@ -206,7 +218,8 @@ template <typename T, int VC, int QT>
 __global__ __launch_bounds__(NT) void grouped_attention_kernel(
     const T* __restrict__ q, const T* __restrict__ cache, const int* __restrict__ tables, int W, int bs,
     const int* __restrict__ row_seq, const int* __restrict__ row_len, float scale, int Hq, int Hkv, int dim, int vdim,
-    int KT, int T_rows, const T* __restrict__ gate, int64_t gate_stride, T* __restrict__ out) {
+    int KT, int T_rows, const T* __restrict__ gate, int64_t gate_stride, T* __restrict__ out,
+    const float* __restrict__ slopes, int chunk, const float* __restrict__ sinks) {
   extern __shared__ float lds[];
   const int Dr = dim + vdim;
   const int KS = Dr + 1;                 // tile row stride (odd: lanes hit distinct banks)
@@ -227,7 +240,7 @@ __global__ __launch_bounds__(NT) void grouped_attention_kernel(
     sQ[e] = (t < T_rows && hh < G) ? ld(q + ((int64_t)t * Hq + g * G + hh) * dim + d) * scale : 0.f;
   }
 
-  int seq_r[QT], len_r[QT];
+  int seq_r[QT], len_r[QT], lo_r[QT];
   bool done[QT];
 #pragma unroll
   for (int r = 0; r < QT; ++r) {
@@ -235,7 +248,11 @@ __global__ __launch_bounds__(NT) void grouped_attention_kernel(
     done[r] = t >= T_rows;
     seq_r[r] = done[r] ? -1 : row_seq[t];
     len_r[r] = done[r] ? 0 : row_len[t];
+    lo_r[r] = (chunk > 0 && len_r[r] > 0) ? ((len_r[r] - 1) / chunk) * chunk : 0;  // first key of the row's chunk
   }
+  const float slope = (slopes != nullptr && head_ok) ? slopes[h] : 0.f;
+  const bool has_sink = sinks != nullptr && head_ok;
+  const float sink = has_sink ? sinks[h] : 0.f;
 
   for (int pass = 0; pass < QT; ++pass) {
     int seq = -1;
@@ -244,22 +261,25 @@ __global__ __launch_bounds__(NT) void grouped_attention_kernel(
       if (seq < 0 && !done[r]) seq = seq_r[r];
     if (seq < 0) break;
     bool act[QT];
-    int maxlen = 0;
+    int maxlen = 0, minlo = 0x7fffffff;
 #pragma unroll
     for (int r = 0; r < QT; ++r) {
       act[r] = !done[r] && seq_r[r] == seq;
-      if (act[r]) maxlen = max(maxlen, len_r[r]);
+      if (act[r]) {
+        maxlen = max(maxlen, len_r[r]);
+        minlo = min(minlo, lo_r[r]);
+      }
     }
     float m[QT], l[QT], acc[QT][VC];
 #pragma unroll
     for (int r = 0; r < QT; ++r) {
-      m[r] = -INFINITY;
-      l[r] = 0.f;
+      m[r] = has_sink ? sink : -INFINITY;  // the sink is a score that is already counted
+      l[r] = has_sink ? 1.f : 0.f;
 #pragma unroll
       for (int c = 0; c < VC; ++c) acc[r][c] = 0.f;
     }
     const int* bt = tables + (int64_t)seq * W;
-    for (int k0 = 0; k0 < maxlen; k0 += KT) {
+    for (int k0 = (minlo / KT) * KT; k0 < maxlen; k0 += KT) {
       __syncthreads();  // previous tile fully used (and sQ written, first time)
       for (int e = threadIdx.x; e < KT * dim; e += NT) {  // keys: row-major in the page
         const int j = e / dim, d = e - j * dim;
@@ -280,15 +300,15 @@ __global__ __launch_bounds__(NT) void grouped_attention_kernel(
       if (!head_ok) continue;
 #pragma unroll
       for (int r = 0; r < QT; ++r) {
-        if (!act[r] || k0 >= len_r[r]) continue;
-        const bool valid = lane < KT && k0 + lane < len_r[r];
+        if (!act[r] || k0 >= len_r[r] || k0 + KT <= lo_r[r]) continue;
+        const bool valid = lane < KT && k0 + lane < len_r[r] && k0 + lane >= lo_r[r];
         float s = -INFINITY;
         if (valid) {
           const float* qv = sQ + (r * 4 + wave) * dim;
           const float* kr = sK + lane * KS;
           float a = 0.f;
           for (int d = 0; d < dim; ++d) a += qv[d] * kr[d];
-          s = a;
+          s = a - slope * (float)(len_r[r] - 1 - (k0 + lane));
         }
         const float mn = fmaxf(m[r], wave_max(s));
         const float corr = expf(m[r] - mn);  // exp(-inf) = 0 on the first tile
@@ -298,7 +318,7 @@ __global__ __launch_bounds__(NT) void grouped_attention_kernel(
 #pragma unroll
         for (int c = 0; c < VC; ++c) acc[r][c] *= corr;
         const int nk = min(KT, len_r[r] - k0);
-        for (int j = 0; j < nk; ++j) {
+        for (int j = max(0, lo_r[r] - k0); j < nk; ++j) {
           const float pj = __shfl(p, j, 64);
           const float* vr = sK + j * KS + dim;
 #pragma unroll
@@ -344,7 +364,8 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache, const int* __restrict__ tables, int W, int bs,
     const int* __restrict__ items, const int* __restrict__ row_len, float scale, int Hq, int Hkv, int dim, int vdim,
     const bf16_t* __restrict__ gate, int64_t gate_stride, bf16_t* __restrict__ out, int split_keys,
-    float* __restrict__ part_o, float* __restrict__ part_ml) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, const float* __restrict__ slopes, int chunk,
+    const float* __restrict__ sinks) {
   constexpr int DkP = 32 * NKS, VP = 16 * NCB;
   constexpr int KS = DkP + 8, VS = MKT + 8;  // LDS row strides (bf16), 16-byte multiples
   // Two tile buffers for the small forms: the next tile is written while the current one is read and
@@ -359,7 +380,8 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r16 = lane & 15, kq = lane >> 4;
   // this lane's query rows (as the B operand's column): item row 16 (4 rb + wave) + r16
-  int mytok[RB], myhead[RB], mylen[RB];
+  int mytok[RB], myhead[RB], mylen[RB], mylo[RB];
+  float myslope[RB];  // in base 2, like the scores
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const int myrow = (rb * 4 + wave) * 16 + r16;
@@ -367,8 +389,12 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
     mytok[rb] = tok0 + (ok ? myrow / G : 0);
     myhead[rb] = g * G + (ok ? myrow % G : 0);
     mylen[rb] = ok ? row_len[mytok[rb]] : 0;
+    mylo[rb] = (chunk > 0 && mylen[rb] > 0) ? ((mylen[rb] - 1) / chunk) * chunk : 0;  // first key of the row's chunk
+    myslope[rb] = slopes ? slopes[myhead[rb]] * 1.44269504088896341f : 0.f;
   }
   const int maxlen = row_len[tok0 + ntok - 1];  // the run's last token sees the most keys
+  // the run's first token starts the earliest chunk; tiles start at multiples of 32 from position 0
+  const int kbase = chunk > 0 ? ((((row_len[tok0] - 1) / chunk) * chunk) / MKT) * MKT : 0;
 
   // padding columns of the key tile and padding rows of the value tile stay zero for the whole kernel
   for (int e = threadIdx.x; e < NBUF * MKT * KS; e += NT) sK[e] = 0;
@@ -390,8 +416,10 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
   float m[RB], l[RB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    m[rb] = -INFINITY;
-    l[rb] = 0.f;
+    // a sink is a score that is already counted (by the first key range only)
+    const bool sk = sinks != nullptr && blockIdx.z == 0;
+    m[rb] = sk ? sinks[myhead[rb]] * 1.44269504088896341f : -INFINITY;
+    l[rb] = sk ? 1.f : 0.f;
 #pragma unroll
     for (int n = 0; n < NCB; ++n) o[rb][n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
@@ -403,7 +431,7 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
 
   // decode steps split a row's keys over blockIdx.z: this workgroup takes [kbeg, kend)
   const int nsplit = gridDim.z;
-  const int kbeg = nsplit > 1 ? blockIdx.z * split_keys : 0;
+  const int kbeg = nsplit > 1 ? kbase + blockIdx.z * split_keys : kbase;
   const int kend = nsplit > 1 ? min(maxlen, kbeg + split_keys) : maxlen;
   constexpr int CK = DkP / 8;                      // 16-byte chunks per key row (padded)
   constexpr int NCK = (MKT * CK + NT - 1) / NT;    // key chunks per thread
@@ -521,8 +549,12 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          sc[rb][kb][r] = (k0 + kb * 16 + kq * 4 + r < min(mylen[rb], kend)) ? a[rb][r] * scale2 : -INFINITY;
+        for (int r = 0; r < 4; ++r) {
+          const int key = k0 + kb * 16 + kq * 4 + r;
+          sc[rb][kb][r] = (key < min(mylen[rb], kend) && key >= mylo[rb])
+                              ? a[rb][r] * scale2 - myslope[rb] * (float)(mylen[rb] - 1 - key)
+                              : -INFINITY;
+        }
     }
     // The weights never pass through LDS. After S^T = K Q^T this lane holds, for its query row r16,
     // the keys 4 kq .. 4 kq + 3 of both 16-key halves of the tile - eight keys, which is exactly one
@@ -672,7 +704,8 @@ __global__ __launch_bounds__(NT) void grouped_attention_merge_kernel(
 template <typename T, int VC>
 int launch_attn(const void* q, const void* cache, const int* tables, int W, int bs, const int* row_seq,
                 const int* row_len, float scale, int Hq, int Hkv, int dim, int vdim, int T_rows, int QT,
-                const void* gate, int64_t gate_stride, void* out, hipStream_t stream) {
+                const void* gate, int64_t gate_stride, void* out, const float* slopes, int chunk, const float* sinks,
+                hipStream_t stream) {
   const int Dr = dim + vdim;
   int KT = 64;
   while (KT > 16 && ((size_t)KT * (Dr + 1) + (size_t)QT * 4 * dim) * 4 > 128 * 1024) KT >>= 1;
@@ -683,7 +716,7 @@ int launch_attn(const void* q, const void* cache, const int* tables, int W, int 
   auto go = [&](auto kern) {
     if (lds > 64 * 1024) (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(kern, grid, dim3(NT), lds, stream, (const T*)q, (const T*)cache, tables, W, bs, row_seq, row_len,
-                       scale, Hq, Hkv, dim, vdim, KT, T_rows, (const T*)gate, gate_stride, (T*)out);
+                       scale, Hq, Hkv, dim, vdim, KT, T_rows, (const T*)gate, gate_stride, (T*)out, slopes, chunk, sinks);
   };
   if (QT == 4) go(grouped_attention_kernel<T, VC, 4>);
   else go(grouped_attention_kernel<T, VC, 1>);
@@ -697,7 +730,7 @@ extern "C" {
 void sm_qkv_rope_cache(const void* qkv, int64_t stride, const float* bias, const int64_t* positions,
                        const float* cos_sin, int Hq, int Hkv, int dim, int vdim, int rot_dims, int interleaved,
                        int unit, float eps, float* v_first, int v_mode, float lam, const int64_t* slots, void* cache,
-                       int bs, void* q_out, int T, int f32, hipStream_t stream) {
+                       int bs, void* q_out, const float* qk_w, int T, int f32, hipStream_t stream) {
   if (T == 0) return;
   // workgroups per token: all heads in parallel for small steps, fewer as the step grows
   const int per_tok = (Hq + Hkv + NT / 64 - 1) / (NT / 64);
@@ -706,7 +739,7 @@ void sm_qkv_rope_cache(const void* qkv, int64_t stride, const float* bias, const
   if (f32)
     hipLaunchKernelGGL((qkv_rope_cache_kernel<float>), grid, dim3(NT), 0, stream, (const float*)qkv, stride, bias,
                        positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit, eps, v_first, v_mode, lam,
-                       slots, (float*)cache, bs, (float*)q_out);
+                       slots, (float*)cache, bs, (float*)q_out, qk_w);
   else if (dim % 8 == 0 && dim <= 512 && ((dim >> 3) & ((dim >> 3) - 1)) == 0 && stride % 8 == 0 &&
            rot_dims % (interleaved ? 8 : 16) == 0 &&
            (((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)cache | (uintptr_t)bias | (uintptr_t)cos_sin) & 15) == 0) {
@@ -716,22 +749,23 @@ void sm_qkv_rope_cache(const void* qkv, int64_t stride, const float* bias, const
     const dim3 vgrid(T, std::max(1, std::min(per_tok_v, 4096 / T)));
     hipLaunchKernelGGL(qkv_rope_cache_vec_kernel, vgrid, dim3(NT), 0, stream, (const bf16_t*)qkv, stride, bias, positions,
                        cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit, eps, v_first, v_mode, lam, slots,
-                       (bf16_t*)cache, bs, (bf16_t*)q_out);
+                       (bf16_t*)cache, bs, (bf16_t*)q_out, qk_w);
   } else
     hipLaunchKernelGGL((qkv_rope_cache_kernel<bf16_t>), grid, dim3(NT), 0, stream, (const bf16_t*)qkv, stride, bias,
                        positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit, eps, v_first, v_mode, lam,
-                       slots, (bf16_t*)cache, bs, (bf16_t*)q_out);
+                       slots, (bf16_t*)cache, bs, (bf16_t*)q_out, qk_w);
 }
 
 // Returns 0, or 1 when the sizes do not fit the kernel (vdim > 1024 or rows too wide for LDS).
 int sm_grouped_attention(const void* q, const void* cache, const int* tables, int W, int bs, const int* row_seq,
                          const int* row_len, float scale, int Hq, int Hkv, int dim, int vdim, int T, int QT,
-                         const void* gate, int64_t gate_stride, void* out, int f32, hipStream_t stream) {
+                         const void* gate, int64_t gate_stride, void* out, int f32, const float* slopes, int chunk,
+                         const float* sinks, hipStream_t stream) {
   if (T == 0) return 0;
   const int vc = (vdim + 63) / 64;
 #define SM_GO(TYPE, VC)                                                                                          \
   return launch_attn<TYPE, VC>(q, cache, tables, W, bs, row_seq, row_len, scale, Hq, Hkv, dim, vdim, T, QT, gate, \
-                               gate_stride, out, stream)
+                               gate_stride, out, slopes, chunk, sinks, stream)
   if (f32) {
     if (vc <= 1) SM_GO(float, 1);
     if (vc <= 2) SM_GO(float, 2);
@@ -755,7 +789,8 @@ int sm_grouped_attention(const void* q, const void* cache, const int* tables, in
 int sm_grouped_attention_mfma(const void* q, const void* cache, const int* tables, int W, int bs, const int* items,
                               int n_items, const int* row_len, float scale, int Hq, int Hkv, int dim, int vdim,
                               const void* gate, int64_t gate_stride, void* out, int nsplit, int split_keys,
-                              float* part_o, float* part_ml, int rb, hipStream_t stream) {
+                              float* part_o, float* part_ml, int rb, const float* slopes, int chunk,
+                              const float* sinks, hipStream_t stream) {
   if (n_items == 0) return 0;
   const int nks = (dim + 31) / 32, ncb = (vdim + 15) / 16;
   if (Hq / Hkv > 64 || nks > 8 || ncb > 16 || (rb != 1 && rb != 2) || (nsplit > 1 && rb != 1) || bs % 8) return 1;
@@ -764,7 +799,8 @@ int sm_grouped_attention_mfma(const void* q, const void* cache, const int* table
 #define SM_GO(NKS, NCB, RB)                                                                                       \
   hipLaunchKernelGGL((grouped_attention_mfma_kernel<NKS, NCB, RB>), grid, dim3(NT), 0, stream, (const bf16_t*)q,   \
                      (const bf16_t*)cache, tables, W, bs, items, row_len, scale, Hq, Hkv, dim, vdim,               \
-                     (const bf16_t*)gate, gate_stride, (bf16_t*)out, split_keys, part_o, part_ml)
+                     (const bf16_t*)gate, gate_stride, (bf16_t*)out, split_keys, part_o, part_ml, slopes, chunk, \
+                     sinks)
 #define SM_GO2(NKS, NCB) \
   if (rb == 2) SM_GO(NKS, NCB, 2); \
   else SM_GO(NKS, NCB, 1)

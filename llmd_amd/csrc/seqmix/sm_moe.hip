@@ -25,7 +25,8 @@ namespace {
 constexpr int TM = 64, TN = 64, TK = 16;
 
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int E, int k,
-                                                        int* __restrict__ ids, float* __restrict__ w, int T) {
+                                                        int* __restrict__ ids, float* __restrict__ w, int T,
+                                                        int sigmoid) {
   const int t = blockIdx.x * 256 + threadIdx.x;
   if (t >= T) return;
   const float* z = logits + (int64_t)t * E;
@@ -46,6 +47,10 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     oi[j] = bi;
     ow[j] = best;
   }
+  if (sigmoid) {  // every chosen logit's own sigmoid
+    for (int j = 0; j < k; ++j) ow[j] = 1.f / (1.f + expf(-ow[j]));
+    return;
+  }
   const float m = ow[0];  // the first chosen is the largest
   float s = 0.f;
   for (int j = 0; j < k; ++j) {
@@ -59,7 +64,8 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
 // One wave per token, lanes over experts (E <= 512: up to 8 logits per lane in registers): k rounds
 // of a wave-wide arg-max over the logits not yet chosen, ties to the lower index.
 __global__ __launch_bounds__(256) void moe_route_wave_kernel(const float* __restrict__ logits, int E, int k,
-                                                             int* __restrict__ ids, float* __restrict__ w, int T) {
+                                                             int* __restrict__ ids, float* __restrict__ w, int T,
+                                                             int sigmoid) {
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (t >= T) return;
@@ -94,7 +100,7 @@ __global__ __launch_bounds__(256) void moe_route_wave_kernel(const float* __rest
       }
     }
     if (j == 0) m0 = best;
-    const float p = expf(best - m0);
+    const float p = sigmoid ? 1.f / (1.f + expf(-best)) : expf(best - m0);
     sum += p;
     if (lane == j) {
       mine = p;
@@ -104,7 +110,7 @@ __global__ __launch_bounds__(256) void moe_route_wave_kernel(const float* __rest
   }
   if (lane < k) {
     ids[(int64_t)t * k + lane] = mine_id;
-    w[(int64_t)t * k + lane] = mine / sum;
+    w[(int64_t)t * k + lane] = sigmoid ? mine : mine / sum;
   }
 }
 
@@ -265,17 +271,20 @@ template <typename T, int ACT>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ A, int64_t a_stride, int kdiv,
                                                        const int* __restrict__ slot_row,
                                                        const int* __restrict__ tile_e, const T* __restrict__ Wt,
-                                                       int N, int K, T* __restrict__ Cout) {
+                                                       int N, int K, T* __restrict__ Cout,
+                                                       const float* __restrict__ row_w) {
   const int e = tile_e[blockIdx.x];
   if (e < 0) return;
   __shared__ float sA[TK][TM + 4], sB[TK][TN + 4];
   __shared__ int srow[TM];
+  __shared__ float sw[TM];  // the row's input weight (gated forms with row_w): scales both sums
   const int tid = threadIdx.x;
   constexpr bool GATED = ACT >= 2;
   const int slot0 = blockIdx.x * TM, n0 = blockIdx.y * (GATED ? TN / 2 : TN);
   if (tid < TM) {
     const int p = slot_row[slot0 + tid];
     srow[tid] = p < 0 ? -1 : (kdiv > 0 ? p / kdiv : slot0 + tid);
+    sw[tid] = (row_w != nullptr && p >= 0) ? row_w[p] : 1.f;
   }
   __syncthreads();
   const T* We = Wt + (int64_t)e * (GATED ? 2 * N : N) * K;
@@ -316,7 +325,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ A, 
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const int n = n0 + tx * 2 + j;
-        if (n < N) st(Cout + (int64_t)(slot0 + r) * N + n, gate_act_<ACT>(acc[i][j]) * acc[i][j + 2]);
+        if (n < N) st(Cout + (int64_t)(slot0 + r) * N + n, gate_act_<ACT>(sw[r] * acc[i][j]) * (sw[r] * acc[i][j + 2]));
       }
       continue;
     }
@@ -352,7 +361,8 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __rest
                                                             const int* __restrict__ slot_row,
                                                             const int* __restrict__ tile_e,
                                                             const bf16_t* __restrict__ Wt, int N, int K,
-                                                            bf16_t* __restrict__ Cout) {
+                                                            bf16_t* __restrict__ Cout,
+                                                            const float* __restrict__ row_w) {
   const int e = tile_e[blockIdx.x];
   if (e < 0) return;
   constexpr bool GATED = ACT >= 2;
@@ -360,12 +370,14 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __rest
   __shared__ __attribute__((aligned(16))) bf16_t sA[TM * MLS];
   __shared__ __attribute__((aligned(16))) bf16_t sB[MBN * MLS];
   __shared__ int srow[TM];
+  __shared__ float sw[TM];  // the row's input weight (gated forms with row_w): scales both sums
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave & 1, wn = wave >> 1;
   const int slot0 = blockIdx.x * TM, n0 = blockIdx.y * (GATED ? MBN / 2 : MBN);
   if (tid < TM) {
     const int p = slot_row[slot0 + tid];
     srow[tid] = p < 0 ? -1 : (kdiv > 0 ? p / kdiv : slot0 + tid);
+    sw[tid] = (row_w != nullptr && p >= 0) ? row_w[p] : 1.f;
   }
   __syncthreads();
   const bf16_t* We = Wt + (int64_t)e * (GATED ? 2 * N : N) * K;
@@ -447,7 +459,9 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __rest
 #pragma unroll
         for (int j = 0; j < NJ / 2; ++j) {
           const int n = n0 + wn * 8 * NJ + j * 16 + r16;
-          if (n < N) st(Cout + (int64_t)(slot0 + row) * N + n, gate_act_<ACT>(acc[i][j][r]) * acc[i][j + NJ / 2][r]);
+          if (n < N)
+            st(Cout + (int64_t)(slot0 + row) * N + n,
+               gate_act_<ACT>(sw[row] * acc[i][j][r]) * (sw[row] * acc[i][j + NJ / 2][r]));
         }
         continue;
       }
@@ -472,7 +486,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const T* __restrict__ 
     for (int j = 0; j < k; ++j) {
       const int slot = pair_slot[t * k + j];
       // slot < 0: an identity expert returns the token's own input
-      s += w[t * k + j] * (slot >= 0 ? ld(y + (int64_t)slot * d + c) : ld(h + t * d + c));
+      s += (w ? w[t * k + j] : 1.f) * (slot >= 0 ? ld(y + (int64_t)slot * d + c) : ld(h + t * d + c));
     }
     st(out + t * d + c, s);
   }
@@ -488,7 +502,7 @@ __global__ __launch_bounds__(256) void moe_combine_vec_kernel(const bf16_t* __re
     float s[8] = {};
     for (int j = 0; j < k; ++j) {
       const int slot = pair_slot[t * k + j];
-      const float wj = w[t * k + j];
+      const float wj = w ? w[t * k + j] : 1.f;
       const u32x4_t v = *reinterpret_cast<const u32x4_t*>(slot >= 0 ? y + (int64_t)slot * d + c : h + t * d + c);
 #pragma unroll
       for (int q = 0; q < 8; ++q) s[q] += wj * __uint_as_float((v[q >> 1] >> (16 * (q & 1))) << 16);
@@ -507,13 +521,15 @@ __global__ __launch_bounds__(256) void moe_combine_vec_kernel(const bf16_t* __re
 
 extern "C" {
 
-void sm_moe_route(const float* logits, int E, int k, int* ids, float* w, int T, hipStream_t stream) {
+// sigmoid: the weights are the chosen logits' sigmoids instead of the softmax over the chosen logits.
+void sm_moe_route(const float* logits, int E, int k, int* ids, float* w, int T, int sigmoid, hipStream_t stream) {
   if (T == 0) return;
   if (E <= 512 && k <= 64) {
-    hipLaunchKernelGGL(moe_route_wave_kernel, dim3((T + 3) / 4), dim3(256), 0, stream, logits, E, k, ids, w, T);
+    hipLaunchKernelGGL(moe_route_wave_kernel, dim3((T + 3) / 4), dim3(256), 0, stream, logits, E, k, ids, w, T,
+                       sigmoid);
     return;
   }
-  hipLaunchKernelGGL(moe_route_kernel, dim3((T + 255) / 256), dim3(256), 0, stream, logits, E, k, ids, w, T);
+  hipLaunchKernelGGL(moe_route_kernel, dim3((T + 255) / 256), dim3(256), 0, stream, logits, E, k, ids, w, T, sigmoid);
 }
 
 void sm_moe_route_scores(const float* logits, const float* corr, int E, int k, int* ids, float* w, int T,
@@ -536,8 +552,11 @@ void sm_moe_group(const int* ids, int n, int E, int* slot_row, int* tile_e, int*
 
 // act: 0 none, 1 erf-GELU, 2 tanh-GELU(gate) * up, 3 SiLU(gate) * up. N = output columns (the gated
 // forms read a weight of 2 N rows per expert).
+// row_w (gated forms): fp32 weight per (token, choice) pair that scales the row's INPUT, applied to
+// both fp32 sums before the activation; nullptr = 1.
 void sm_moe_gemm(const void* A, int64_t a_stride, int kdiv, const int* slot_row, const int* tile_e, const void* W,
-                 int N, int K, void* C, int max_tiles, int rows_hint, int act, int f32, hipStream_t stream) {
+                 int N, int K, void* C, int max_tiles, int rows_hint, int act, int f32, const float* row_w,
+                 hipStream_t stream) {
   const bool gated = act >= 2;
   if (!f32 && K % 8 == 0 && a_stride % 8 == 0 && ((uintptr_t)A & 15) == 0 && ((uintptr_t)W & 15) == 0) {
     // wide tiles when the step has prompt-sized row counts (most tiles are full) and N is wide
@@ -546,7 +565,7 @@ void sm_moe_gemm(const void* A, int64_t a_stride, int kdiv, const int* slot_row,
     const dim3 g2(max_tiles, (N + mbn - 1) / mbn);
 #define SM_MF(A_, NJ)                                                                                          \
   hipLaunchKernelGGL((moe_gemm_mfma_kernel<A_, NJ>), g2, dim3(256), 0, stream, (const bf16_t*)A, a_stride, kdiv, \
-                     slot_row, tile_e, (const bf16_t*)W, N, K, (bf16_t*)C)
+                     slot_row, tile_e, (const bf16_t*)W, N, K, (bf16_t*)C, row_w)
 #define SM_MF2(A_) \
   if (wide) SM_MF(A_, 8); \
   else SM_MF(A_, 4)
@@ -562,7 +581,7 @@ void sm_moe_gemm(const void* A, int64_t a_stride, int kdiv, const int* slot_row,
   const dim3 grid(max_tiles, (N + tn - 1) / tn);
 #define SM_GO(TYPE, A_)                                                                                         \
   hipLaunchKernelGGL((moe_gemm_kernel<TYPE, A_>), grid, dim3(256), 0, stream, (const TYPE*)A, a_stride, kdiv,   \
-                     slot_row, tile_e, (const TYPE*)W, N, K, (TYPE*)C)
+                     slot_row, tile_e, (const TYPE*)W, N, K, (TYPE*)C, row_w)
 #define SM_GO2(TYPE)                   \
   if (act == 0) SM_GO(TYPE, 0);        \
   else if (act == 1) SM_GO(TYPE, 1);   \
