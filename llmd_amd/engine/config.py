@@ -399,6 +399,23 @@ def _tiny_negunex() -> ModelConfig:
 _register(_tiny_negunex())
 
 
+def _tiny_zumizen() -> ModelConfig:
+    left = {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 16, "scale": 32 ** -0.5, "mask": {"size": 48}}
+    right = {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 32, "conv": 4}
+    experts = {"kind": "moe", "expert": {"ff": 64}, "router": {"experts": 6, "top": 2}}
+    return zumizen_config({
+        "architecture": "Zumizen", "name": "tiny-zumizen", "width": 128, "vocab": 512, "norm": {"eps": 1e-6},
+        "embedding": {"scale": 1.0, "bigram": {"buckets": 251, "mul_prev": 31, "mul_cur": 7}}, "logit_softcap": 30.0,
+        "max_position": 4096, "eos": 1,
+        "layers": [{"type": "channel_delta", "mixer": dict(right, decay_rank=8, gate_rank=16), "mlp": experts},
+                   {"type": "parallel", "mlp": experts,
+                    "mixer": {"left": left, "right": right, "left_scale": 1.0, "right_scale": 1.0}},
+                   {"type": "channel_delta", "mixer": dict(right, kv_heads=4, decay_rank=8, gate_rank=16), "mlp": None}]})
+
+
+_register(_tiny_zumizen())
+
+
 def get_model_config(name_or_path: str) -> ModelConfig:
     if name_or_path in PRESETS:
         return dataclasses.replace(PRESETS[name_or_path])

@@ -294,17 +294,18 @@ def moe_gated_ffn(h, ids, w, w1, w2, kind, scale_input=False):
 def bigram_embed(ids, table, scale, bigram, buckets, mul_prev, mul_cur, prev_state, seq_start, seq_slot, seq_init,
                  x, out_dtype):
     x.copy_(table[ids].float() * scale)
-    if bigram is not None:
-        rows = torch.empty_like(ids)
-        for i in range(seq_slot.numel()):
-            lo, hi, sl = int(seq_start[i]), int(seq_start[i + 1]), int(seq_slot[i])
-            if hi == lo:
-                continue
+    rows = torch.empty_like(ids)
+    for i in range(seq_slot.numel()):
+        lo, hi, sl = int(seq_start[i]), int(seq_start[i + 1]), int(seq_slot[i])
+        if hi == lo:
+            continue
+        if bigram is not None:
             prev = torch.cat([prev_state[sl].view(1).long(), ids[lo:hi - 1]])
             rows[lo:hi] = (prev * mul_prev + ids[lo:hi] * mul_cur) % buckets
             if not int(seq_init[i]):
                 rows[lo] = buckets
-            prev_state[sl] = ids[hi - 1]
+        prev_state[sl] = ids[hi - 1]
+    if bigram is not None:
         x.add_(bigram[rows].float())
     return x.to(out_dtype)
 

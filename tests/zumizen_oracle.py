@@ -215,12 +215,12 @@ def random_weights(cfg, seed=0, dtype=torch.float32):
         vec(pre + "A_log", H, mean=-0.5, std=0.5)
         vec(pre + "norm", dv)
         if channel:
-            r = m.get("rank", 8)
-            mat(pre + "a1", r, d)
-            mat(pre + "a2", H * dk, r)
+            ra, rg = m.get("rank", 8), m.get("rank", 8) + 3   # two sizes that only the tensors give
+            mat(pre + "a1", ra, d)
+            mat(pre + "a2", H * dk, ra)
             vec(pre + "dt_bias", H * dk, mean=0.0, std=0.5)
-            mat(pre + "g1", r, d)
-            mat(pre + "g2", H * dv, r)
+            mat(pre + "g1", rg, d)
+            mat(pre + "g2", H * dv, rg)
         else:
             mat(pre + "a", H, d)
             vec(pre + "dt_bias", H, mean=0.0, std=0.5)
