@@ -50,9 +50,11 @@ void sm_bigram_embed(const int64_t*, const void*, float, int64_t, const void*, i
                      const int*, const int*, const int*, const int*, int*, float*, void*, int, int, int, hipStream_t);
 void sm_post_norm_add(const void*, int64_t, const void*, int64_t, float, float, const float*, const void*, float*, float,
                       const void*, void*, int, int, int, hipStream_t);
+int sm_gated_delta_rows(int);
 int sm_gated_delta_scan(const void*, int64_t, int, int, int, int, const void*, int64_t, const void*, int64_t, int,
                         const float*, const float*, const void*, int64_t, int, const void*, float, float*, const int*,
-                        const int*, const int*, void*, int, int, hipStream_t);
+                        const int*, const int*, void*, float*, float*, float*, float*, float*, int, int, int,
+                        hipStream_t);
 void sm_moe_combine(const void*, const int*, const float*, int, int, void*, const void*, int, int, hipStream_t);
 }
 
@@ -654,13 +656,20 @@ void gated_delta_scan(Tensor xc, int64_t G, int64_t dk, int64_t H, int64_t dv, T
               "state [slots, H, dk, dv]");
   check_seq(seq_start, seq_slot, seq_init, state.size(0));
   TORCH_CHECK(out.is_contiguous() && out.dim() == 2 && out.size(0) == T && out.size(1) == H * dv, "out [T, H dv]");
+  const int64_t KD = sm_gated_delta_rows(dk);
+  TORCH_CHECK(KD > 0, "gated_delta_scan: key size above 256");
+  TORCH_CHECK(seq_slot.numel() <= 65535, "too many sequences in a step");
+  // fp32 workspaces of the three kernels: [qn | kn | dec | beta | o_raw]
+  const int64_t n_qk = T * G * KD, n_dec = per_channel ? T * H * KD : T * H, n_b = T * H, n_o = T * H * dv;
+  Tensor ws = torch::empty({2 * n_qk + n_dec + n_b + n_o + 4}, torch::dtype(torch::kFloat32).device(xc.device()));
+  float* w0 = ws.data_ptr<float>();
   const int rc = sm_gated_delta_scan(
       xc.data_ptr(), xc.stride(0), G, dk, H, dv, beta_raw.data_ptr(), beta_raw.stride(0), decay_raw.data_ptr(),
       decay_raw.stride(0), per_channel ? 1 : 0, A.data_ptr<float>(), dt_bias.data_ptr<float>(), gate_raw.data_ptr(),
       gate_raw.stride(0), gate_sigmoid ? 1 : 0, norm_w.data_ptr(), (float)eps, state.data_ptr<float>(),
-      seq_start.data_ptr<int>(), seq_slot.data_ptr<int>(), seq_init.data_ptr<int>(), out.data_ptr(), seq_slot.numel(),
-      is_f32(xc), cur());
-  TORCH_CHECK(rc == 0, "gated_delta_scan: head sizes above 256");
+      seq_start.data_ptr<int>(), seq_slot.data_ptr<int>(), seq_init.data_ptr<int>(), out.data_ptr(), w0, w0 + n_qk,
+      w0 + 2 * n_qk, w0 + 2 * n_qk + n_dec, w0 + 2 * n_qk + n_dec + n_b, T, seq_slot.numel(), is_f32(xc), cur());
+  TORCH_CHECK(rc == 0, "gated_delta_scan: key size above 256");
 }
 
 }  // namespace

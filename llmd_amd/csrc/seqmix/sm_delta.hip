@@ -7,168 +7,180 @@
 //   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
 //   out = o / rms(o) * norm_w * gate,  gate = silu or sigmoid of its input
 //
-// One workgroup per (value head, sequence): CT column threads (a multiple of 64 >= dv) x NW key
-// groups. Thread (g, j) keeps the KR = KD / NW key rows [g KR, (g + 1) KR) of column j of S in
-// registers (KD >= dk, padded rows stay zero). Per token the first dk threads compute the key-side
-// vectors (unit key, unit query, decay) in fp32 and broadcast them through LDS; every group forms its
-// part of S^T k and, after the update, of S^T q, and the parts meet in LDS. The inputs of a block of
-// TB tokens are fetched while the previous block runs.
+// Only the recurrence is sequential, so it is all the scan kernel does. A first kernel, parallel
+// over the tokens, makes the unit queries and keys, the decays and beta (fp32, rows padded to
+// KD = 4 KR with q = k = 0 and g = 1); a last one, parallel again, norms the read-outs and applies
+// the gate. The columns of S never meet in the recurrence, so the scan has no barrier: a workgroup
+// is ONE wave that owns 16 value columns of one head and sequence, lane = (column c, row group r),
+// and keeps rows [r KR, (r + 1) KR) of its column in registers. The two sums over the key
+// rows (S^T k and S^T q) end with two quad exchanges between the four lanes of a column. The next
+// token's inputs are loaded while the current token computes.
 #include "seqmix_common.h"
+#include <algorithm>
 
 using namespace sm;
 
 namespace {
 
-// Two sums over a workgroup of BT threads in one pass; every thread gets both.
-template <int BT>
-__device__ __forceinline__ void block_sum2(float& a, float& b, float* red) {
-  a = wave_sum(a);
-  b = wave_sum(b);
-  if ((threadIdx.x & 63) == 0) {
-    red[(threadIdx.x >> 6) * 2] = a;
-    red[(threadIdx.x >> 6) * 2 + 1] = b;
-  }
-  __syncthreads();
-  float sa = 0.f, sb = 0.f;
+constexpr int NT = 256;
+
+// Unit queries and keys, decays and beta of every token (fp32). qn, kn [T, G, KD]; dec [T, H, KD]
+// (one decay per key channel) or [T, H]; beta [T, H]. Rows beyond dk: q = k = 0, g = 1.
+template <typename T>
+__global__ __launch_bounds__(NT) void delta_prep_kernel(const T* __restrict__ xc, int64_t x_stride, int G, int dk,
+                                                       int KD, int H, const T* __restrict__ beta_raw,
+                                                       int64_t beta_stride, const T* __restrict__ decay_raw,
+                                                       int64_t decay_stride, int per_channel,
+                                                       const float* __restrict__ A, const float* __restrict__ dt_bias,
+                                                       float* __restrict__ qn, float* __restrict__ kn,
+                                                       float* __restrict__ dec, float* __restrict__ beta) {
+  const int64_t t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const T* xr = xc + t * x_stride;
+  const float qscale = 1.f / sqrtf((float)dk);
+  for (int hd = wave; hd < 2 * G; hd += NT / 64) {  // q heads, then k heads: back to back in the row
+    float r[4], ss = 0.f;                           // KD <= 256
 #pragma unroll
-  for (int i = 0; i < BT / 64; ++i) {
-    sa += red[2 * i];
-    sb += red[2 * i + 1];
+    for (int i = 0; i < 4; ++i) {
+      const int e = lane + 64 * i;
+      r[i] = e < dk ? ld(xr + hd * dk + e) : 0.f;
+      ss += r[i] * r[i];
+    }
+    const float inv = Fn<T>::rsqrt(wave_sum(ss) + 1e-6f) * (hd < G ? qscale : 1.f);
+    float* dst = (hd < G ? qn + (t * G + hd) * KD : kn + (t * G + hd - G) * KD);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int e = lane + 64 * i;
+      if (e < KD) dst[e] = r[i] * inv;
+    }
   }
-  __syncthreads();
-  a = sa;
-  b = sb;
+  if (per_channel) {
+    for (int idx = threadIdx.x; idx < H * KD; idx += NT) {
+      const int h = idx / KD, i = idx - h * KD;
+      float g = 1.f;
+      if (i < dk) g = Fn<T>::exp(-A[h] * Fn<T>::softplus(ld(decay_raw + t * decay_stride + h * dk + i) + dt_bias[h * dk + i]));
+      dec[t * H * KD + idx] = g;
+    }
+  }
+  for (int h = threadIdx.x; h < H; h += NT) {
+    if (!per_channel) dec[t * H + h] = Fn<T>::exp(-A[h] * Fn<T>::softplus(ld(decay_raw + t * decay_stride + h) + dt_bias[h]));
+    beta[t * H + h] = Fn<T>::sigmoid(ld(beta_raw + t * beta_stride + h));
+  }
 }
 
-template <typename T, int KD, int CT, int NW>
-__global__ __launch_bounds__(CT * NW) void gated_delta_scan_kernel(
-    const T* __restrict__ xc, int64_t x_stride, int G, int dk, int H, int dv, const T* __restrict__ beta_raw,
-    int64_t beta_stride, const T* __restrict__ decay_raw, int64_t decay_stride, int per_channel,
-    const float* __restrict__ A, const float* __restrict__ dt_bias, const T* __restrict__ gate_raw,
-    int64_t gate_stride, int gate_sigmoid, const T* __restrict__ norm_w, float eps, float* __restrict__ state,
-    const int* __restrict__ seq_start, const int* __restrict__ seq_slot, const int* __restrict__ seq_init,
-    T* __restrict__ out) {
-  constexpr int BT = CT * NW, KR = KD / NW;
-  __shared__ __attribute__((aligned(16))) float sk[KD], sq[KD], sg[KD];
-  __shared__ float part[NW][CT];
-  __shared__ float red[2 * (BT / 64)];
-  const int h = blockIdx.x, s = blockIdx.y;
-  const int tid = threadIdx.x;
-  const int j = tid % CT, g = tid / CT;
-  const bool col = j < dv;
-  const bool keyl = tid < dk;                 // this thread owns key channel tid of the token
-  const bool lead = g == 0 && col;            // this thread writes column j of the output
-  const int qh = h / (H / G);                 // the query / key head of this value head
+// Sum over the four lanes of a quad (lanes 4 c .. 4 c + 3): two DPP exchanges, no LDS.
+__device__ __forceinline__ float quad_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));  // 1 0 3 2
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));  // 2 3 0 1
+  return v;
+}
+
+// The recurrence. One wave per (head, block of 16 value columns, sequence). CH: a decay per key row.
+// PF: the next token's inputs are fetched ahead into a second set of registers.
+template <typename T, int KR, bool CH, bool PF>
+__global__ __launch_bounds__(64) void gated_delta_scan_kernel(
+    const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ dec,
+    const float* __restrict__ beta, const T* __restrict__ xc, int64_t x_stride, int voff, int G, int dk, int H, int dv,
+    float* __restrict__ state, const int* __restrict__ seq_start, const int* __restrict__ seq_slot,
+    const int* __restrict__ seq_init, float* __restrict__ o_raw) {
+  constexpr int KD = 4 * KR;
+  const int ncb = (dv + 15) >> 4;
+  const int h = blockIdx.x / ncb, cb = blockIdx.x - h * ncb, s = blockIdx.y;
+  const int lane = threadIdx.x, r = lane & 3, c = lane >> 2;
+  const int col = cb * 16 + c;
+  const bool colok = col < dv;
+  const int qh = h / (H / G);
+  const int row0 = r * KR;
   const int lo = seq_start[s], hi = seq_start[s + 1];
+  if (lo >= hi) return;
   float* sp = state + ((int64_t)seq_slot[s] * H + h) * dk * dv;
-  const int i0 = g * KR;
-  float S[KR];
   const bool init = seq_init[s] != 0;
+  float S[KR];
 #pragma unroll
-  for (int i = 0; i < KR; ++i) S[i] = (col && i0 + i < dk && init) ? sp[(int64_t)(i0 + i) * dv + j] : 0.f;
-  for (int i = dk + tid; i < KD; i += BT) {
-    sk[i] = sq[i] = 0.f;
-    sg[i] = 1.f;
-  }
-  const float Ah = A[h];
-  const int dch = per_channel ? h * dk + (keyl ? tid : 0) : h;  // this thread's decay column
-  const float dtb = dt_bias[dch];
-  const float nwj = col ? ld(norm_w + j) : 0.f;
-  const float qscale = 1.f / sqrtf((float)dk);
-  const int nqk = G * dk;
-  constexpr int TB = 4;
-  float nq[TB], nk[TB], na[TB], nv[TB], nb[TB], ng[TB];
-  auto fetch = [&](int t0) {
-#pragma unroll
-    for (int b = 0; b < TB; ++b) {
-      nq[b] = nk[b] = na[b] = nv[b] = ng[b] = 0.f;
-      const int t = min(t0 + b, hi - 1);  // past the end: a valid row, never used
-      const T* xr = xc + (int64_t)t * x_stride;
-      nb[b] = ld(beta_raw + (int64_t)t * beta_stride + h);
-      if (keyl) {
-        nq[b] = ld(xr + qh * dk + tid);
-        nk[b] = ld(xr + nqk + qh * dk + tid);
-        na[b] = ld(decay_raw + (int64_t)t * decay_stride + dch);
-      }
-      if (col) nv[b] = ld(xr + 2 * nqk + h * dv + j);
-      if (lead) ng[b] = ld(gate_raw + (int64_t)t * gate_stride + h * dv + j);
-    }
+  for (int i = 0; i < KR; ++i) S[i] = (init && colok && row0 + i < dk) ? sp[(int64_t)(row0 + i) * dv + col] : 0.f;
+  struct In {
+    float k[KR], q[KR], g[CH ? KR : 1], b, v;
   };
-  if (lo < hi) fetch(lo);
-  for (int t0 = lo; t0 < hi; t0 += TB) {
-    float cq[TB], ck[TB], ca[TB], cv[TB], cb[TB], cg[TB];
+  auto fetch = [&](In& in, int t) {
+    const float4* kp = reinterpret_cast<const float4*>(kn + ((int64_t)t * G + qh) * KD + row0);
+    const float4* qp = reinterpret_cast<const float4*>(qn + ((int64_t)t * G + qh) * KD + row0);
 #pragma unroll
-    for (int b = 0; b < TB; ++b) {
-      cq[b] = nq[b];
-      ck[b] = nk[b];
-      ca[b] = na[b];
-      cv[b] = nv[b];
-      cb[b] = nb[b];
-      cg[b] = ng[b];
+    for (int i = 0; i < KR; i += 4) {
+      const float4 a = kp[i >> 2], b = qp[i >> 2];
+      in.k[i] = a.x; in.k[i + 1] = a.y; in.k[i + 2] = a.z; in.k[i + 3] = a.w;
+      in.q[i] = b.x; in.q[i + 1] = b.y; in.q[i + 2] = b.z; in.q[i + 3] = b.w;
     }
-    if (t0 + TB < hi) fetch(t0 + TB);
-#pragma unroll
-    for (int b = 0; b < TB; ++b) {
-      const int t = t0 + b;
-      if (t >= hi) break;
-      float ssq = keyl ? cq[b] * cq[b] : 0.f, ssk = keyl ? ck[b] * ck[b] : 0.f;
-      block_sum2<BT>(ssq, ssk, red);  // also fences the previous token's LDS reads
-      if (keyl) {
-        sq[tid] = cq[b] * Fn<T>::rsqrt(ssq + 1e-6f) * qscale;
-        sk[tid] = ck[b] * Fn<T>::rsqrt(ssk + 1e-6f);
-        sg[tid] = Fn<T>::exp(-Ah * Fn<T>::softplus(ca[b] + dtb));
-      }
-      __syncthreads();
-      // the key-side vectors come as 16-byte LDS broadcasts; entries beyond dk are 0 (decay 1)
-      float pred = 0.f;
+    if (CH) {
+      const float4* gp = reinterpret_cast<const float4*>(dec + ((int64_t)t * H + h) * KD + row0);
 #pragma unroll
       for (int i = 0; i < KR; i += 4) {
-        const float4 g4 = *reinterpret_cast<const float4*>(&sg[i0 + i]);
-        const float4 k4 = *reinterpret_cast<const float4*>(&sk[i0 + i]);
-        S[i] *= g4.x;
-        S[i + 1] *= g4.y;
-        S[i + 2] *= g4.z;
-        S[i + 3] *= g4.w;
-        pred += k4.x * S[i] + k4.y * S[i + 1] + k4.z * S[i + 2] + k4.w * S[i + 3];
+        const float4 a = gp[i >> 2];
+        in.g[i] = a.x; in.g[i + 1] = a.y; in.g[i + 2] = a.z; in.g[i + 3] = a.w;
       }
-      if (NW > 1) {
-        part[g][j] = pred;
-        __syncthreads();
-        pred = 0.f;
+    } else {
+      in.g[0] = dec[(int64_t)t * H + h];
+    }
+    in.b = beta[(int64_t)t * H + h];
+    in.v = colok ? ld(xc + (int64_t)t * x_stride + voff + h * dv + col) : 0.f;
+  };
+  auto step = [&](const In& in, int t) {
+    float p[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int q = 0; q < NW; ++q) pred += part[q][j];
-        __syncthreads();
-      }
-      const float u = Fn<T>::sigmoid(cb[b]) * (cv[b] - pred);
-      float o = 0.f;
+    for (int i = 0; i < KR; ++i) {
+      S[i] *= CH ? in.g[i] : in.g[0];
+      p[i & 3] += in.k[i] * S[i];
+    }
+    const float pred = quad_sum((p[0] + p[1]) + (p[2] + p[3]));
+    const float u = in.b * (in.v - pred);
+    float o[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < KR; i += 4) {
-        const float4 k4 = *reinterpret_cast<const float4*>(&sk[i0 + i]);
-        const float4 q4 = *reinterpret_cast<const float4*>(&sq[i0 + i]);
-        S[i] += k4.x * u;
-        S[i + 1] += k4.y * u;
-        S[i + 2] += k4.z * u;
-        S[i + 3] += k4.w * u;
-        o += S[i] * q4.x + S[i + 1] * q4.y + S[i + 2] * q4.z + S[i + 3] * q4.w;
-      }
-      if (NW > 1) {
-        part[g][j] = o;
-        __syncthreads();
-        o = 0.f;
-#pragma unroll
-        for (int q = 0; q < NW; ++q) o += part[q][j];
-      }
-      const float ss = block_sum<BT>(lead ? o * o : 0.f, red);
-      if (lead) {
-        const float gt = gate_sigmoid ? Fn<T>::sigmoid(cg[b]) : Fn<T>::silu(cg[b]);
-        st(out + (int64_t)t * H * dv + h * dv + j, o * Fn<T>::rsqrt(ss / (float)dv + eps) * nwj * gt);
-      }
+    for (int i = 0; i < KR; ++i) {
+      S[i] += in.k[i] * u;
+      o[i & 3] += S[i] * in.q[i];
+    }
+    const float ov = quad_sum((o[0] + o[1]) + (o[2] + o[3]));
+    if (r == 0 && colok) o_raw[(int64_t)t * H * dv + h * dv + col] = ov;
+  };
+  if (PF) {
+    In cur, nxt;
+    fetch(cur, lo);
+    for (int t = lo; t < hi; ++t) {
+      if (t + 1 < hi) fetch(nxt, t + 1);
+      step(cur, t);
+      cur = nxt;
+    }
+  } else {
+    for (int t = lo; t < hi; ++t) {
+      In cur;
+      fetch(cur, t);
+      step(cur, t);
     }
   }
-  if (col && hi > lo) {
+  if (colok) {
 #pragma unroll
     for (int i = 0; i < KR; ++i)
-      if (i0 + i < dk) sp[(int64_t)(i0 + i) * dv + j] = S[i];
+      if (row0 + i < dk) sp[(int64_t)(row0 + i) * dv + col] = S[i];
+  }
+}
+
+// out = o / rms(o) * norm_w * gate per head; a wave per (token, head), any dv.
+template <typename T>
+__global__ __launch_bounds__(NT) void delta_out_kernel(const float* __restrict__ o_raw, const T* __restrict__ gate_raw,
+                                                      int64_t gate_stride, int gate_sigmoid,
+                                                      const T* __restrict__ norm_w, float eps, int H, int dv,
+                                                      T* __restrict__ out) {
+  const int64_t t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int h = blockIdx.y * (NT / 64) + wave; h < H; h += gridDim.y * (NT / 64)) {
+    const float* orow = o_raw + (t * H + h) * dv;
+    float ss = 0.f;
+    for (int e = lane; e < dv; e += 64) ss += orow[e] * orow[e];
+    const float inv = Fn<T>::rsqrt(wave_sum(ss) / (float)dv + eps);
+    for (int e = lane; e < dv; e += 64) {
+      const float gr = ld(gate_raw + t * gate_stride + h * dv + e);
+      const float gt = gate_sigmoid ? Fn<T>::sigmoid(gr) : Fn<T>::silu(gr);
+      st(out + (t * H + h) * dv + e, orow[e] * inv * ld(norm_w + e) * gt);
+    }
   }
 }
 
@@ -176,33 +188,43 @@ __global__ __launch_bounds__(CT * NW) void gated_delta_scan_kernel(
 
 extern "C" {
 
-// Returns 0, or 1 when a head size does not fit (dk > 256 or dv > 256).
+// Padded key rows per head (4 KR) for a key size, or 0 when it does not fit (dk > 256).
+int sm_gated_delta_rows(int dk) { return dk <= 32 ? 32 : dk <= 64 ? 64 : dk <= 128 ? 128 : dk <= 256 ? 256 : 0; }
+
+// Workspaces (fp32): qn, kn [T, G, KD]; dec [T, H, KD] or [T, H]; beta [T, H]; o_raw [T, H, dv].
+// Returns 0, or 1 when the key size does not fit (dk > 256).
 int sm_gated_delta_scan(const void* xc, int64_t x_stride, int G, int dk, int H, int dv, const void* beta_raw,
                         int64_t beta_stride, const void* decay_raw, int64_t decay_stride, int per_channel,
                         const float* A, const float* dt_bias, const void* gate_raw, int64_t gate_stride,
                         int gate_sigmoid, const void* norm_w, float eps, float* state, const int* seq_start,
-                        const int* seq_slot, const int* seq_init, void* out, int nseq, int f32, hipStream_t stream) {
-  if (nseq == 0) return 0;
-  if (dk > 256 || dv > 256) return 1;
-  const dim3 grid(H, nseq);
-#define SM_GO(TYPE, KD, CT, NW)                                                                                     \
-  hipLaunchKernelGGL((gated_delta_scan_kernel<TYPE, KD, CT, NW>), grid, dim3(CT * NW), 0, stream, (const TYPE*)xc,   \
-                     x_stride, G, dk, H, dv, (const TYPE*)beta_raw, beta_stride, (const TYPE*)decay_raw,             \
-                     decay_stride, per_channel, A, dt_bias, (const TYPE*)gate_raw, gate_stride, gate_sigmoid,        \
-                     (const TYPE*)norm_w, eps, state, seq_start, seq_slot, seq_init, (TYPE*)out)
-#define SM_KD(TYPE, CT, NW)                    \
-  if (dk <= 32) SM_GO(TYPE, 32, CT, NW);       \
-  else if (dk <= 64) SM_GO(TYPE, 64, CT, NW);  \
-  else if (dk <= 128) SM_GO(TYPE, 128, CT, NW); \
-  else SM_GO(TYPE, 256, CT, NW)
-#define SM_CT(TYPE)                       \
-  if (dv <= 64) { SM_KD(TYPE, 64, 4); }   \
-  else if (dv <= 128) { SM_KD(TYPE, 128, 2); } \
-  else { SM_KD(TYPE, 256, 2); }
-  if (f32) { SM_CT(float) }
-  else { SM_CT(bf16_t) }
-#undef SM_CT
-#undef SM_KD
+                        const int* seq_slot, const int* seq_init, void* out, float* qn, float* kn, float* dec,
+                        float* beta, float* o_raw, int T, int nseq, int f32, hipStream_t stream) {
+  if (nseq == 0 || T == 0) return 0;
+  const int KD = sm_gated_delta_rows(dk);
+  if (KD == 0) return 1;
+  const int voff = 2 * G * dk;
+  const dim3 grid(H * ((dv + 15) / 16), nseq);
+  const dim3 ogrid(T, std::max(1, std::min((H + 3) / 4, 4096 / T)));
+#define SM_GO(TYPE, KR, CH)                                                                                        \
+  hipLaunchKernelGGL((gated_delta_scan_kernel<TYPE, KR, CH, (KR <= 32)>), grid, dim3(64), 0, stream, qn, kn, dec,    \
+                     beta, (const TYPE*)xc, x_stride, voff, G, dk, H, dv, state, seq_start, seq_slot, seq_init, o_raw)
+#define SM_KR(TYPE, CH)                   \
+  if (KD == 32) SM_GO(TYPE, 8, CH);       \
+  else if (KD == 64) SM_GO(TYPE, 16, CH); \
+  else if (KD == 128) SM_GO(TYPE, 32, CH); \
+  else SM_GO(TYPE, 64, CH)
+#define SM_ALL(TYPE)                                                                                                \
+  hipLaunchKernelGGL((delta_prep_kernel<TYPE>), dim3(T), dim3(NT), 0, stream, (const TYPE*)xc, x_stride, G, dk, KD, \
+                     H, (const TYPE*)beta_raw, beta_stride, (const TYPE*)decay_raw, decay_stride, per_channel, A,   \
+                     dt_bias, qn, kn, dec, beta);                                                                   \
+  if (per_channel) { SM_KR(TYPE, true); }                                                                           \
+  else { SM_KR(TYPE, false); }                                                                                      \
+  hipLaunchKernelGGL((delta_out_kernel<TYPE>), ogrid, dim3(NT), 0, stream, o_raw, (const TYPE*)gate_raw,            \
+                     gate_stride, gate_sigmoid, (const TYPE*)norm_w, eps, H, dv, (TYPE*)out)
+  if (f32) { SM_ALL(float); }
+  else { SM_ALL(bf16_t); }
+#undef SM_ALL
+#undef SM_KR
 #undef SM_GO
   return 0;
 }

@@ -19,6 +19,15 @@ hyper-connected streams) run beside the existing models of the same layer geomet
   negunex-moe   : width 2048, 32 heads / 4 kv heads x 128, 128 experts + 4 identity, 8 chosen, ff 768 -
                   beside Qwen3-30B-A3B layers (models/moe_llama.py)
 
+Two Zumizen stacks (post-norm residual, bigram embedding, experts whose score scales their input):
+
+  zumizen-channel  : width 2048, gated delta rule 32 heads x 64 (key) x 64 (value) with a decay per key
+                     channel, 4 taps; 64 experts, 6 chosen, ff 1408 - beside Mekusun's ``delta``
+                     (same heads and sizes) and ``latent+moe`` (same experts)
+  zumizen-parallel : width 2048, chunked attention 32 heads / 4 kv heads x 128 (chunks of 1024, distance
+                     bias, sink) beside a gated delta rule 16 heads / 8 q-k heads x 128 x 128; 128 experts,
+                     8 chosen, ff 768 - beside ``negunex-moe`` (same attention and expert geometry)
+
 Prefill: one prompt of ``--tokens`` tokens in one step. Decode: ``--batch`` sequences with that
 context, one token each. One JSON line with tokens/s and ms per layer for every entry.
 """
@@ -69,6 +78,28 @@ def _negunex(width, heads, kv, ff=None, experts=None):
     return lambda n: negunex_config({"architecture": "Negunex", "width": width, "vocab": 32000, "streams": 2,
                                      "norm": {"eps": 1e-6},
                                      "layers": [{"type": "attention", "mixer": mixer, "mlp": mlp}] * n})
+
+
+def _zumizen(kind: str):
+    from llmd_amd.engine.config import zumizen_config
+
+    if kind == "channel":
+        layer = {"type": "channel_delta",
+                 "mixer": {"heads": 32, "kv_heads": 32, "dim": 64, "vdim": 64, "conv": 4, "decay_rank": 64,
+                           "gate_rank": 64},
+                 "mlp": {"kind": "moe", "expert": {"ff": 1408}, "router": {"experts": 64, "top": 6}}}
+    else:
+        layer = {"type": "parallel",
+                 "mixer": {"left": {"heads": 32, "kv_heads": 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                                    "mask": {"size": 1024}},
+                           "right": {"heads": 16, "kv_heads": 8, "dim": 128, "vdim": 128, "conv": 4},
+                           "left_scale": 1.0, "right_scale": 1.0},
+                 "mlp": {"kind": "moe", "expert": {"ff": 768}, "router": {"experts": 128, "top": 8}}}
+    return lambda n: zumizen_config({"architecture": "Zumizen", "name": "zumizen-" + kind, "width": WIDTH,
+                                     "vocab": 32000, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+                                     "embedding": {"scale": 1.0,
+                                                   "bigram": {"buckets": 65521, "mul_prev": 31337, "mul_cur": 7919}},
+                                     "layers": [layer] * n})
 
 
 def _runner(mc, tokens: int, batch: int, device: str):
@@ -134,7 +165,9 @@ def run(tokens: int = 2048, batch: int = 32, n_layers: int = 4, reps: int = 5, d
                                                       vocab_size=32000, name="llama-3-8b-cut"), n_layers),
             ("negunex-moe", _negunex(2048, 32, 4, experts=(128, 8, 768))(n_layers), n_layers),
             ("qwen3-30b-a3b layers", dataclasses.replace(get_model_config("qwen3-30b-a3b"), num_hidden_layers=n_layers,
-                                                         vocab_size=32000, name="qwen3-30b-a3b-cut"), n_layers)]
+                                                         vocab_size=32000, name="qwen3-30b-a3b-cut"), n_layers),
+            ("zumizen-channel", _zumizen("channel")(n_layers), n_layers),
+            ("zumizen-parallel", _zumizen("parallel")(n_layers), n_layers)]
     for name, mc, L in todo:
         if only and not any(name.startswith(o) for o in only.split(",")):
             continue
