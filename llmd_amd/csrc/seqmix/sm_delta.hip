@@ -13,8 +13,8 @@
 // the gate. The columns of S never meet in the recurrence, so the scan has no barrier: a workgroup
 // is ONE wave that owns 16 value columns of one head and sequence, lane = (column c, row group r),
 // and keeps rows [r KR, (r + 1) KR) of its column in registers. The two sums over the key
-// rows (S^T k and S^T q) end with two quad exchanges between the four lanes of a column. The next
-// token's inputs are loaded while the current token computes.
+// rows (S^T k and S^T q) end with two quad exchanges between the four lanes of a column. The
+// key-side vectors reach the wave in blocks of tokens through LDS, fetched a block ahead.
 #include "seqmix_common.h"
 #include <algorithm>
 
@@ -76,14 +76,20 @@ __device__ __forceinline__ float quad_sum(float v) {
 }
 
 // The recurrence. One wave per (head, block of 16 value columns, sequence). CH: a decay per key row.
-// PF: the next token's inputs are fetched ahead into a second set of registers.
-template <typename T, int KR, bool CH, bool PF>
+// The key-side vectors of TB tokens at a time go through LDS: while the wave computes one block of
+// tokens from one buffer, the next block's loads are in flight into registers, and are written to the
+// other buffer afterwards - the recurrence never waits for global memory. Per token a lane reads its
+// KR rows of k, q (and g) as 16-byte LDS broadcasts.
+template <typename T, int KR, bool CH, int TB>
 __global__ __launch_bounds__(64) void gated_delta_scan_kernel(
     const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ dec,
     const float* __restrict__ beta, const T* __restrict__ xc, int64_t x_stride, int voff, int G, int dk, int H, int dv,
     float* __restrict__ state, const int* __restrict__ seq_start, const int* __restrict__ seq_slot,
     const int* __restrict__ seq_init, float* __restrict__ o_raw) {
-  constexpr int KD = 4 * KR;
+  constexpr int KD = 4 * KR, NV = CH ? 3 : 2;       // vectors per token: k, q (, g)
+  constexpr int C4 = KD / 4;                         // 16-byte chunks per vector
+  constexpr int NL = TB * NV * C4 / 64;              // chunks per lane and block (KD >= 32: a whole number)
+  __shared__ __attribute__((aligned(16))) float buf[2][TB * NV * KD];
   const int ncb = (dv + 15) >> 4;
   const int h = blockIdx.x / ncb, cb = blockIdx.x - h * ncb, s = blockIdx.y;
   const int lane = threadIdx.x, r = lane & 3, c = lane >> 2;
@@ -98,63 +104,94 @@ __global__ __launch_bounds__(64) void gated_delta_scan_kernel(
   float S[KR];
 #pragma unroll
   for (int i = 0; i < KR; ++i) S[i] = (init && colok && row0 + i < dk) ? sp[(int64_t)(row0 + i) * dv + col] : 0.f;
-  struct In {
-    float k[KR], q[KR], g[CH ? KR : 1], b, v;
-  };
-  auto fetch = [&](In& in, int t) {
-    const float4* kp = reinterpret_cast<const float4*>(kn + ((int64_t)t * G + qh) * KD + row0);
-    const float4* qp = reinterpret_cast<const float4*>(qn + ((int64_t)t * G + qh) * KD + row0);
+  float4 stage[NL];
+  float vb[TB], bb[TB], gb[CH ? 1 : TB];            // the block's values, betas and per-head decays
+  auto fetch = [&](int t0) {                          // block t0 .. t0 + TB - 1 -> registers
 #pragma unroll
-    for (int i = 0; i < KR; i += 4) {
-      const float4 a = kp[i >> 2], b = qp[i >> 2];
-      in.k[i] = a.x; in.k[i + 1] = a.y; in.k[i + 2] = a.z; in.k[i + 3] = a.w;
-      in.q[i] = b.x; in.q[i + 1] = b.y; in.q[i + 2] = b.z; in.q[i + 3] = b.w;
+    for (int n = 0; n < NL; ++n) {
+      const int e = lane + 64 * n;
+      const int j = e / (NV * C4), rem = e - j * (NV * C4);
+      const int var = rem / C4, i4 = rem - var * C4;
+      const int64_t t = t0 + j;
+      float4 v4 = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (t < hi) {                                   // a short run (one decoded token) loads only what it has
+        const float* src =
+            var == 0 ? kn + (t * G + qh) * KD : var == 1 ? qn + (t * G + qh) * KD : dec + (t * H + h) * KD;
+        v4 = reinterpret_cast<const float4*>(src)[i4];
+      }
+      stage[n] = v4;
     }
-    if (CH) {
-      const float4* gp = reinterpret_cast<const float4*>(dec + ((int64_t)t * H + h) * KD + row0);
+#pragma unroll
+    for (int j = 0; j < TB; ++j) {
+      const int64_t t = t0 + j;
+      vb[j] = bb[j] = 0.f;
+      if (!CH) gb[j] = 1.f;
+      if (t >= hi) continue;
+      vb[j] = colok ? ld(xc + t * x_stride + voff + h * dv + col) : 0.f;
+      bb[j] = beta[t * H + h];
+      if (!CH) gb[j] = dec[t * H + h];
+    }
+  };
+  auto spill = [&](int which) {                       // registers -> LDS buffer
+#pragma unroll
+    for (int n = 0; n < NL; ++n) reinterpret_cast<float4*>(buf[which])[lane + 64 * n] = stage[n];
+  };
+  fetch(lo);
+  spill(0);
+  __syncthreads();
+  int which = 0;
+  for (int t0 = lo; t0 < hi; t0 += TB, which ^= 1) {
+    float cv[TB], cbeta[TB], cg[CH ? 1 : TB];
+#pragma unroll
+    for (int j = 0; j < TB; ++j) {
+      cv[j] = vb[j];
+      cbeta[j] = bb[j];
+      if (!CH) cg[j] = gb[j];
+    }
+    const bool more = t0 + TB < hi;
+    if (more) fetch(t0 + TB);
+    const float* bk = buf[which];
+#pragma unroll
+    for (int j = 0; j < TB; ++j) {
+      const int t = t0 + j;
+      if (t >= hi) break;
+      const float4* kp = reinterpret_cast<const float4*>(bk + (j * NV + 0) * KD + row0);
+      const float4* qp = reinterpret_cast<const float4*>(bk + (j * NV + 1) * KD + row0);
+      const float4* gp = reinterpret_cast<const float4*>(bk + (j * NV + (CH ? 2 : 0)) * KD + row0);
+      float k[KR];
+      float p[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int i = 0; i < KR; i += 4) {
-        const float4 a = gp[i >> 2];
-        in.g[i] = a.x; in.g[i + 1] = a.y; in.g[i + 2] = a.z; in.g[i + 3] = a.w;
+        const float4 k4 = kp[i >> 2];
+        k[i] = k4.x; k[i + 1] = k4.y; k[i + 2] = k4.z; k[i + 3] = k4.w;
+        if (CH) {
+          const float4 g4 = gp[i >> 2];
+          S[i] *= g4.x; S[i + 1] *= g4.y; S[i + 2] *= g4.z; S[i + 3] *= g4.w;
+        } else {
+          S[i] *= cg[j]; S[i + 1] *= cg[j]; S[i + 2] *= cg[j]; S[i + 3] *= cg[j];
+        }
+        p[0] += k[i] * S[i];
+        p[1] += k[i + 1] * S[i + 1];
+        p[2] += k[i + 2] * S[i + 2];
+        p[3] += k[i + 3] * S[i + 3];
       }
-    } else {
-      in.g[0] = dec[(int64_t)t * H + h];
-    }
-    in.b = beta[(int64_t)t * H + h];
-    in.v = colok ? ld(xc + (int64_t)t * x_stride + voff + h * dv + col) : 0.f;
-  };
-  auto step = [&](const In& in, int t) {
-    float p[4] = {0.f, 0.f, 0.f, 0.f};
+      const float pred = quad_sum((p[0] + p[1]) + (p[2] + p[3]));
+      const float u = cbeta[j] * (cv[j] - pred);
+      float o[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int i = 0; i < KR; ++i) {
-      S[i] *= CH ? in.g[i] : in.g[0];
-      p[i & 3] += in.k[i] * S[i];
+      for (int i = 0; i < KR; i += 4) {
+        const float4 q4 = qp[i >> 2];
+        S[i] += k[i] * u; S[i + 1] += k[i + 1] * u; S[i + 2] += k[i + 2] * u; S[i + 3] += k[i + 3] * u;
+        o[0] += S[i] * q4.x;
+        o[1] += S[i + 1] * q4.y;
+        o[2] += S[i + 2] * q4.z;
+        o[3] += S[i + 3] * q4.w;
+      }
+      const float ov = quad_sum((o[0] + o[1]) + (o[2] + o[3]));
+      if (r == 0 && colok) o_raw[(int64_t)t * H * dv + h * dv + col] = ov;
     }
-    const float pred = quad_sum((p[0] + p[1]) + (p[2] + p[3]));
-    const float u = in.b * (in.v - pred);
-    float o[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int i = 0; i < KR; ++i) {
-      S[i] += in.k[i] * u;
-      o[i & 3] += S[i] * in.q[i];
-    }
-    const float ov = quad_sum((o[0] + o[1]) + (o[2] + o[3]));
-    if (r == 0 && colok) o_raw[(int64_t)t * H * dv + h * dv + col] = ov;
-  };
-  if (PF) {
-    In cur, nxt;
-    fetch(cur, lo);
-    for (int t = lo; t < hi; ++t) {
-      if (t + 1 < hi) fetch(nxt, t + 1);
-      step(cur, t);
-      cur = nxt;
-    }
-  } else {
-    for (int t = lo; t < hi; ++t) {
-      In cur;
-      fetch(cur, t);
-      step(cur, t);
-    }
+    if (more) spill(which ^ 1);
+    __syncthreads();  // one wave: orders the buffer's writes before the next block's reads
   }
   if (colok) {
 #pragma unroll
@@ -206,7 +243,7 @@ int sm_gated_delta_scan(const void* xc, int64_t x_stride, int G, int dk, int H, 
   const dim3 grid(H * ((dv + 15) / 16), nseq);
   const dim3 ogrid(T, std::max(1, std::min((H + 3) / 4, 4096 / T)));
 #define SM_GO(TYPE, KR, CH)                                                                                        \
-  hipLaunchKernelGGL((gated_delta_scan_kernel<TYPE, KR, CH, (KR <= 32)>), grid, dim3(64), 0, stream, qn, kn, dec,    \
+  hipLaunchKernelGGL((gated_delta_scan_kernel<TYPE, KR, CH, (KR <= 32 ? 16 : 8)>), grid, dim3(64), 0, stream, qn, kn, dec, \
                      beta, (const TYPE*)xc, x_stride, voff, G, dk, H, dv, state, seq_start, seq_slot, seq_init, o_raw)
 #define SM_KR(TYPE, CH)                   \
   if (KD == 32) SM_GO(TYPE, 8, CH);       \
