@@ -104,94 +104,109 @@ __global__ __launch_bounds__(64) void gated_delta_scan_kernel(
   float S[KR];
 #pragma unroll
   for (int i = 0; i < KR; ++i) S[i] = (init && colok && row0 + i < dk) ? sp[(int64_t)(row0 + i) * dv + col] : 0.f;
-  float4 stage[NL];
-  float vb[TB], bb[TB], gb[CH ? 1 : TB];            // the block's values, betas and per-head decays
-  auto fetch = [&](int t0) {                          // block t0 .. t0 + TB - 1 -> registers
+  // one token: kp, qp, gp point at this lane's KR rows of k, q and (CH) g; returns the read-out
+  auto token = [&](const float4* kp, const float4* qp, const float4* gp, float gj, float bj, float vj) {
+    float k[KR];
+    float p[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int n = 0; n < NL; ++n) {
-      const int e = lane + 64 * n;
-      const int j = e / (NV * C4), rem = e - j * (NV * C4);
-      const int var = rem / C4, i4 = rem - var * C4;
-      const int64_t t = t0 + j;
-      float4 v4 = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (t < hi) {                                   // a short run (one decoded token) loads only what it has
-        const float* src =
-            var == 0 ? kn + (t * G + qh) * KD : var == 1 ? qn + (t * G + qh) * KD : dec + (t * H + h) * KD;
-        v4 = reinterpret_cast<const float4*>(src)[i4];
+    for (int i = 0; i < KR; i += 4) {
+      const float4 k4 = kp[i >> 2];
+      k[i] = k4.x; k[i + 1] = k4.y; k[i + 2] = k4.z; k[i + 3] = k4.w;
+      if (CH) {
+        const float4 g4 = gp[i >> 2];
+        S[i] *= g4.x; S[i + 1] *= g4.y; S[i + 2] *= g4.z; S[i + 3] *= g4.w;
+      } else {
+        S[i] *= gj; S[i + 1] *= gj; S[i + 2] *= gj; S[i + 3] *= gj;
       }
-      stage[n] = v4;
+      p[0] += k[i] * S[i];
+      p[1] += k[i + 1] * S[i + 1];
+      p[2] += k[i + 2] * S[i + 2];
+      p[3] += k[i + 3] * S[i + 3];
     }
+    const float pred = quad_sum((p[0] + p[1]) + (p[2] + p[3]));
+    const float u = bj * (vj - pred);
+    float o[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < TB; ++j) {
-      const int64_t t = t0 + j;
-      vb[j] = bb[j] = 0.f;
-      if (!CH) gb[j] = 1.f;
-      if (t >= hi) continue;
-      vb[j] = colok ? ld(xc + t * x_stride + voff + h * dv + col) : 0.f;
-      bb[j] = beta[t * H + h];
-      if (!CH) gb[j] = dec[t * H + h];
+    for (int i = 0; i < KR; i += 4) {
+      const float4 q4 = qp[i >> 2];
+      S[i] += k[i] * u; S[i + 1] += k[i + 1] * u; S[i + 2] += k[i + 2] * u; S[i + 3] += k[i + 3] * u;
+      o[0] += S[i] * q4.x;
+      o[1] += S[i + 1] * q4.y;
+      o[2] += S[i + 2] * q4.z;
+      o[3] += S[i + 3] * q4.w;
     }
+    return quad_sum((o[0] + o[1]) + (o[2] + o[3]));
   };
-  auto spill = [&](int which) {                       // registers -> LDS buffer
-#pragma unroll
-    for (int n = 0; n < NL; ++n) reinterpret_cast<float4*>(buf[which])[lane + 64 * n] = stage[n];
-  };
-  fetch(lo);
-  spill(0);
-  __syncthreads();
-  int which = 0;
-  for (int t0 = lo; t0 < hi; t0 += TB, which ^= 1) {
-    float cv[TB], cbeta[TB], cg[CH ? 1 : TB];
-#pragma unroll
-    for (int j = 0; j < TB; ++j) {
-      cv[j] = vb[j];
-      cbeta[j] = bb[j];
-      if (!CH) cg[j] = gb[j];
+  if (hi - lo <= 2) {
+    // a decoded token (or two): the lane's rows straight from global memory, no staging
+    for (int64_t t = lo; t < hi; ++t) {
+      const float4* kp = reinterpret_cast<const float4*>(kn + (t * G + qh) * KD + row0);
+      const float4* qp = reinterpret_cast<const float4*>(qn + (t * G + qh) * KD + row0);
+      const float4* gp = reinterpret_cast<const float4*>(CH ? dec + (t * H + h) * KD + row0 : kn);
+      const float vj = colok ? ld(xc + t * x_stride + voff + h * dv + col) : 0.f;
+      const float ov = token(kp, qp, gp, CH ? 1.f : dec[t * H + h], beta[t * H + h], vj);
+      if (r == 0 && colok) o_raw[t * H * dv + h * dv + col] = ov;
     }
-    const bool more = t0 + TB < hi;
-    if (more) fetch(t0 + TB);
-    const float* bk = buf[which];
+  } else {
+    float4 stage[NL];
+    float vb[TB], bb[TB], gb[CH ? 1 : TB];            // the block's values, betas and per-head decays
+    auto fetch = [&](int t0) {                          // block t0 .. t0 + TB - 1 -> registers
 #pragma unroll
-    for (int j = 0; j < TB; ++j) {
-      const int t = t0 + j;
-      if (t >= hi) break;
-      const float4* kp = reinterpret_cast<const float4*>(bk + (j * NV + 0) * KD + row0);
-      const float4* qp = reinterpret_cast<const float4*>(bk + (j * NV + 1) * KD + row0);
-      const float4* gp = reinterpret_cast<const float4*>(bk + (j * NV + (CH ? 2 : 0)) * KD + row0);
-      float k[KR];
-      float p[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int i = 0; i < KR; i += 4) {
-        const float4 k4 = kp[i >> 2];
-        k[i] = k4.x; k[i + 1] = k4.y; k[i + 2] = k4.z; k[i + 3] = k4.w;
-        if (CH) {
-          const float4 g4 = gp[i >> 2];
-          S[i] *= g4.x; S[i + 1] *= g4.y; S[i + 2] *= g4.z; S[i + 3] *= g4.w;
-        } else {
-          S[i] *= cg[j]; S[i + 1] *= cg[j]; S[i + 2] *= cg[j]; S[i + 3] *= cg[j];
+      for (int n = 0; n < NL; ++n) {
+        const int e = lane + 64 * n;
+        const int j = e / (NV * C4), rem = e - j * (NV * C4);
+        const int var = rem / C4, i4 = rem - var * C4;
+        const int64_t t = t0 + j;
+        float4 v4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (t < hi) {
+          const float* src =
+              var == 0 ? kn + (t * G + qh) * KD : var == 1 ? qn + (t * G + qh) * KD : dec + (t * H + h) * KD;
+          v4 = reinterpret_cast<const float4*>(src)[i4];
         }
-        p[0] += k[i] * S[i];
-        p[1] += k[i + 1] * S[i + 1];
-        p[2] += k[i + 2] * S[i + 2];
-        p[3] += k[i + 3] * S[i + 3];
+        stage[n] = v4;
       }
-      const float pred = quad_sum((p[0] + p[1]) + (p[2] + p[3]));
-      const float u = cbeta[j] * (cv[j] - pred);
-      float o[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < KR; i += 4) {
-        const float4 q4 = qp[i >> 2];
-        S[i] += k[i] * u; S[i + 1] += k[i + 1] * u; S[i + 2] += k[i + 2] * u; S[i + 3] += k[i + 3] * u;
-        o[0] += S[i] * q4.x;
-        o[1] += S[i + 1] * q4.y;
-        o[2] += S[i + 2] * q4.z;
-        o[3] += S[i + 3] * q4.w;
+      for (int j = 0; j < TB; ++j) {
+        const int64_t t = t0 + j;
+        vb[j] = bb[j] = 0.f;
+        if (!CH) gb[j] = 1.f;
+        if (t >= hi) continue;
+        vb[j] = colok ? ld(xc + t * x_stride + voff + h * dv + col) : 0.f;
+        bb[j] = beta[t * H + h];
+        if (!CH) gb[j] = dec[t * H + h];
       }
-      const float ov = quad_sum((o[0] + o[1]) + (o[2] + o[3]));
-      if (r == 0 && colok) o_raw[(int64_t)t * H * dv + h * dv + col] = ov;
+    };
+    auto spill = [&](int which) {                       // registers -> LDS buffer
+#pragma unroll
+      for (int n = 0; n < NL; ++n) reinterpret_cast<float4*>(buf[which])[lane + 64 * n] = stage[n];
+    };
+    fetch(lo);
+    spill(0);
+    __syncthreads();
+    int which = 0;
+    for (int t0 = lo; t0 < hi; t0 += TB, which ^= 1) {
+      float cv[TB], cbeta[TB], cg[CH ? 1 : TB];
+#pragma unroll
+      for (int j = 0; j < TB; ++j) {
+        cv[j] = vb[j];
+        cbeta[j] = bb[j];
+        if (!CH) cg[j] = gb[j];
+      }
+      const bool more = t0 + TB < hi;
+      if (more) fetch(t0 + TB);
+      const float* bk = buf[which];
+#pragma unroll
+      for (int j = 0; j < TB; ++j) {
+        if (t0 + j >= hi) break;
+        const float ov = token(reinterpret_cast<const float4*>(bk + (j * NV + 0) * KD + row0),
+                               reinterpret_cast<const float4*>(bk + (j * NV + 1) * KD + row0),
+                               reinterpret_cast<const float4*>(bk + (j * NV + (CH ? 2 : 0)) * KD + row0),
+                               CH ? 1.f : cg[j], cbeta[j], cv[j]);
+        if (r == 0 && colok) o_raw[(int64_t)(t0 + j) * H * dv + h * dv + col] = ov;
+      }
+      if (more) spill(which ^ 1);
+      __syncthreads();  // one wave: orders the buffer's writes before the next block's reads
     }
-    if (more) spill(which ^ 1);
-    __syncthreads();  // one wave: orders the buffer's writes before the next block's reads
   }
   if (colok) {
 #pragma unroll
