@@ -238,7 +238,7 @@ class GroupedAttention(torch.nn.Module):
     gate         multiply the concatenated heads by sigmoid(W_g h) before the output projection
     norm_weight  the unit norms have weights ``q_norm`` / ``k_norm`` [dim], shared by the heads
     slopes       "pow2": the score of query i and key j loses 2^(-8 (h + 1) / heads) * (i - j)
-    chunk        > 0: query i sees only keys j >= (i // chunk) * chunk (chunks from position 0)
+    chunk        > 0: query i sees only keys j >= (i // chunk) * chunk (borders at multiples of chunk in the sequence's positions)
     sink         one more score of 0 per head in the softmax's denominator, without a value
     out_bias     the output projection has a bias
     """

@@ -2,7 +2,9 @@
 scan, the generalized delta rule, zero-centred norms with layer scale, depth averaging, plain
 (ungated) expert feed-forwards; hyper-connected residual streams with layer norm, grouped-query
 attention with its own key and value sizes (bias, rotary, unit norm, value mixing, gate), gated
-activations, score routing with a selection-only correction, gated experts with identity experts.
+activations, score routing with a selection-only correction, gated experts with identity experts;
+the bigram embedding, the post-norm residual add, the gated delta rule, distance slopes / chunks /
+sinks in grouped attention, sigmoid routing with experts whose weight scales their input.
 
 GPU tensors go to the ``llmd_amd._C_seqmix`` library (csrc/seqmix/*.hip, built on its own so a
 model that needs only these kernels compiles only these); it is templated on the activation
@@ -271,8 +273,8 @@ def grouped_attention(q, cache, dim, vdim, scale: float, seq, gate=None, slopes=
     multiplied by sigmoid(gate). Returns [T, Hq * vdim].
 
     ``slopes`` fp32 [Hq]: the score of query i and key j loses slopes[h] * (i - j).
-    ``chunk`` > 0: query i sees key j only inside its own chunk, j >= (i // chunk) * chunk, chunks
-    counted from the sequence's position 0.
+    ``chunk`` > 0: query i sees key j only inside its own chunk, j >= (i // chunk) * chunk; i and j are
+    positions in the sequence, not in the step.
     ``sinks`` fp32 [Hq]: one more score per head in the softmax's denominator, without a value.
 
     bfloat16 runs on the matrix cores (work item = up to 64 (token, head-of-group) rows of one
