@@ -302,9 +302,11 @@ class GroupedAttention(torch.nn.Module):
         """kv_layer [blocks, 1, Hkv, bs, dim + vdim] -> [blocks, Hkv, bs, dim + vdim]."""
         self.cache = kv_layer[:, 0]
 
-    def forward(self, h, meta: AttnMeta, shared=None):
+    def forward(self, h, meta: AttnMeta, shared=None, p=None):
+        """``p``: this layer's projection of h when a caller has already computed it (a row view)."""
         T = h.shape[0]
-        p = self.proj(h)
+        if p is None:
+            p = self.proj(h)
         q = torch.empty(T, self.Hq, self.dim, dtype=h.dtype, device=h.device)
         v_first, mode = None, 0
         if self.v_mix:
@@ -415,9 +417,11 @@ class GatedDeltaMixer(torch.nn.Module):
     def bind_state(self, tensors):
         self.conv_state, self.state = tensors
 
-    def forward(self, h, meta: AttnMeta):
+    def forward(self, h, meta: AttnMeta, p=None):
+        """``p``: this layer's projection of h when a caller has already computed it (a row view)."""
         s = meta.seq
-        p = self.proj(h)
+        if p is None:
+            p = self.proj(h)
         xc = sm.causal_conv_silu(p, self.C, self.conv, self.conv_b, self.conv_state, s.seq_start, s.seq_slot,
                                  s.seq_init, s.max_q)
         c0 = self.C
@@ -441,9 +445,20 @@ class ParallelMixer(torch.nn.Module):
         super().__init__()
         self.left, self.right = left, right
         self.left_scale, self.right_scale = float(left_scale), float(right_scale)
+        # both read the same input: their input projections are the two row ranges of ONE weight (one
+        # GEMM per layer); each mixer's own ``proj.weight`` stays a view of its rows, which is what the
+        # weight loader fills
+        wl, wr = left.proj.weight.data, right.proj.weight.data
+        self.n_left = wl.shape[0]
+        self.proj = ColumnLinear(left.proj.in_f, self.n_left + wr.shape[0], shard=False, device=wl.device,
+                                 dtype=wl.dtype)
+        self.proj.weight.data.copy_(torch.cat([wl, wr]))
+        left.proj.weight = torch.nn.Parameter(self.proj.weight.data[:self.n_left], requires_grad=False)
+        right.proj.weight = torch.nn.Parameter(self.proj.weight.data[self.n_left:], requires_grad=False)
 
     def forward(self, h, meta: AttnMeta):
-        return self.left(h, meta), self.right(h, meta)
+        p = self.proj(h)
+        return self.left(h, meta, p=p[:, :self.n_left]), self.right(h, meta, p=p[:, self.n_left:])
 
 
 class SigmoidMoE(torch.nn.Module):
