@@ -9,12 +9,13 @@
 //
 // Only the recurrence is sequential, so it is all the scan kernel does. A first kernel, parallel
 // over the tokens, makes the unit queries and keys, the decays and beta (fp32, rows padded to
-// KD = 4 KR with q = k = 0 and g = 1); a last one, parallel again, norms the read-outs and applies
+// KD = 32 .. 256 with q = k = 0 and g = 1); a last one, parallel again, norms the read-outs and applies
 // the gate. The columns of S never meet in the recurrence, so the scan has no barrier: a workgroup
-// is ONE wave that owns 16 value columns of one head and sequence, lane = (column c, row group r),
-// and keeps rows [r KR, (r + 1) KR) of its column in registers. The two sums over the key
-// rows (S^T k and S^T q) end with two quad exchanges between the four lanes of a column. The
-// key-side vectors reach the wave in blocks of tokens through LDS, fetched a block ahead.
+// is ONE wave that owns 16 (or 8) value columns of one head and sequence, lane = (column c, row group
+// r of 4 (or 8)), and keeps rows [r KR, (r + 1) KR) of its column in registers. The two sums over the
+// key rows (S^T k and S^T q) end with DPP exchanges between the lanes of a column. The key-side
+// vectors reach the wave in blocks of tokens through LDS, fetched a block ahead. Steps with few
+// (head, sequence) pairs - a prompt - take the 8 x 8 form: twice the waves, half the work of each.
 #include "seqmix_common.h"
 #include <algorithm>
 
@@ -68,32 +69,38 @@ __global__ __launch_bounds__(NT) void delta_prep_kernel(const T* __restrict__ xc
   }
 }
 
-// Sum over the four lanes of a quad (lanes 4 c .. 4 c + 3): two DPP exchanges, no LDS.
-__device__ __forceinline__ float quad_sum(float v) {
+// Sum over the RG (4 or 8) neighbouring lanes of a column (lanes RG c .. RG c + RG - 1): DPP
+// exchanges, no LDS. After the two quad exchanges all four lanes of a quad hold the quad's sum; the
+// mirror inside a half row (lane i <-> 7 - i) then brings the other quad's.
+template <int RG>
+__device__ __forceinline__ float group_sum(float v) {
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));  // 1 0 3 2
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));  // 2 3 0 1
+  if (RG == 8)
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // half mirror
   return v;
 }
 
-// The recurrence. One wave per (head, block of 16 value columns, sequence). CH: a decay per key row.
+// The recurrence. One wave per (head, block of 64 / RG value columns, sequence); RG = 4 or 8 row groups
+// (lanes) per column, KR rows per lane. CH: a decay per key row.
 // The key-side vectors of TB tokens at a time go through LDS: while the wave computes one block of
 // tokens from one buffer, the next block's loads are in flight into registers, and are written to the
 // other buffer afterwards - the recurrence never waits for global memory. Per token a lane reads its
 // KR rows of k, q (and g) as 16-byte LDS broadcasts.
-template <typename T, int KR, bool CH, int TB>
+template <typename T, int KR, int RG, bool CH, int TB>
 __global__ __launch_bounds__(64) void gated_delta_scan_kernel(
     const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ dec,
     const float* __restrict__ beta, const T* __restrict__ xc, int64_t x_stride, int voff, int G, int dk, int H, int dv,
     float* __restrict__ state, const int* __restrict__ seq_start, const int* __restrict__ seq_slot,
     const int* __restrict__ seq_init, float* __restrict__ o_raw) {
-  constexpr int KD = 4 * KR, NV = CH ? 3 : 2;       // vectors per token: k, q (, g)
+  constexpr int KD = RG * KR, CPW = 64 / RG, NV = CH ? 3 : 2;       // vectors per token: k, q (, g)
   constexpr int C4 = KD / 4;                         // 16-byte chunks per vector
   constexpr int NL = TB * NV * C4 / 64;              // chunks per lane and block (KD >= 32: a whole number)
   __shared__ __attribute__((aligned(16))) float buf[2][TB * NV * KD];
-  const int ncb = (dv + 15) >> 4;
+  const int ncb = (dv + CPW - 1) / CPW;
   const int h = blockIdx.x / ncb, cb = blockIdx.x - h * ncb, s = blockIdx.y;
-  const int lane = threadIdx.x, r = lane & 3, c = lane >> 2;
-  const int col = cb * 16 + c;
+  const int lane = threadIdx.x, r = lane % RG, c = lane / RG;
+  const int col = cb * CPW + c;
   const bool colok = col < dv;
   const int qh = h / (H / G);
   const int row0 = r * KR;
@@ -123,7 +130,7 @@ __global__ __launch_bounds__(64) void gated_delta_scan_kernel(
       p[2] += k[i + 2] * S[i + 2];
       p[3] += k[i + 3] * S[i + 3];
     }
-    const float pred = quad_sum((p[0] + p[1]) + (p[2] + p[3]));
+    const float pred = group_sum<RG>((p[0] + p[1]) + (p[2] + p[3]));
     const float u = bj * (vj - pred);
     float o[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -135,7 +142,7 @@ __global__ __launch_bounds__(64) void gated_delta_scan_kernel(
       o[2] += S[i + 2] * q4.z;
       o[3] += S[i + 3] * q4.w;
     }
-    return quad_sum((o[0] + o[1]) + (o[2] + o[3]));
+    return group_sum<RG>((o[0] + o[1]) + (o[2] + o[3]));
   };
   if (hi - lo <= 2) {
     // a decoded token (or two): the lane's rows straight from global memory, no staging
@@ -255,28 +262,37 @@ int sm_gated_delta_scan(const void* xc, int64_t x_stride, int G, int dk, int H, 
   const int KD = sm_gated_delta_rows(dk);
   if (KD == 0) return 1;
   const int voff = 2 * G * dk;
-  const dim3 grid(H * ((dv + 15) / 16), nseq);
+  // 16 columns x 4 row groups per wave when the step brings many waves anyway (decode: 64-byte pieces of
+  // the state's rows); 8 x 8 when it brings few (a prompt): twice the waves, half the work of each
+  const bool wide = (int64_t)nseq * H * ((dv + 15) / 16) >= 1024;
+  const int cpw = wide ? 16 : 8;
+  const dim3 grid(H * ((dv + cpw - 1) / cpw), nseq);
   const dim3 ogrid(T, std::max(1, std::min((H + 3) / 4, 4096 / T)));
-#define SM_GO(TYPE, KR, CH)                                                                                        \
-  hipLaunchKernelGGL((gated_delta_scan_kernel<TYPE, KR, CH, (KR <= 32 ? 16 : 8)>), grid, dim3(64), 0, stream, qn, kn, dec, \
-                     beta, (const TYPE*)xc, x_stride, voff, G, dk, H, dv, state, seq_start, seq_slot, seq_init, o_raw)
-#define SM_KR(TYPE, CH)                   \
-  if (KD == 32) SM_GO(TYPE, 8, CH);       \
-  else if (KD == 64) SM_GO(TYPE, 16, CH); \
-  else if (KD == 128) SM_GO(TYPE, 32, CH); \
-  else SM_GO(TYPE, 64, CH)
+#define SM_GO(TYPE, KR, RG, CH)                                                                                     \
+  hipLaunchKernelGGL((gated_delta_scan_kernel<TYPE, KR, RG, CH, (KR * RG <= 128 ? 16 : 8)>), grid, dim3(64), 0, stream, \
+                     qn, kn, dec, beta, (const TYPE*)xc, x_stride, voff, G, dk, H, dv, state, seq_start, seq_slot,  \
+                     seq_init, o_raw)
+#define SM_RG(TYPE, KD_, CH)              \
+  if (wide) SM_GO(TYPE, KD_ / 4, 4, CH);  \
+  else SM_GO(TYPE, KD_ / 8, 8, CH)
+#define SM_KR(TYPE, CH)                           \
+  if (KD == 32) { SM_RG(TYPE, 32, CH); }          \
+  else if (KD == 64) { SM_RG(TYPE, 64, CH); }     \
+  else if (KD == 128) { SM_RG(TYPE, 128, CH); }   \
+  else { SM_RG(TYPE, 256, CH); }
 #define SM_ALL(TYPE)                                                                                                \
   hipLaunchKernelGGL((delta_prep_kernel<TYPE>), dim3(T), dim3(NT), 0, stream, (const TYPE*)xc, x_stride, G, dk, KD, \
                      H, (const TYPE*)beta_raw, beta_stride, (const TYPE*)decay_raw, decay_stride, per_channel, A,   \
                      dt_bias, qn, kn, dec, beta);                                                                   \
-  if (per_channel) { SM_KR(TYPE, true); }                                                                           \
-  else { SM_KR(TYPE, false); }                                                                                      \
+  if (per_channel) { SM_KR(TYPE, true) }                                                                           \
+  else { SM_KR(TYPE, false) }                                                                                      \
   hipLaunchKernelGGL((delta_out_kernel<TYPE>), ogrid, dim3(NT), 0, stream, o_raw, (const TYPE*)gate_raw,            \
                      gate_stride, gate_sigmoid, (const TYPE*)norm_w, eps, H, dv, (TYPE*)out)
   if (f32) { SM_ALL(float); }
   else { SM_ALL(bf16_t); }
 #undef SM_ALL
 #undef SM_KR
+#undef SM_RG
 #undef SM_GO
   return 0;
 }
