@@ -76,6 +76,8 @@ class ModelConfig:
     hyper_streams: int = 0
     # hashed bigram table added to the embedding (models/zumizen.py): {buckets, mul_prev, mul_cur} or None
     bigram: Optional[dict] = None
+    # taps of the short causal convolution in front of every mixer (models/kakalorn.py), 1 = none
+    conv_taps: int = 1
     name: str = "custom"
 
     def __post_init__(self):
@@ -123,6 +125,8 @@ class ModelConfig:
             return mekusun_config(d, shapes) if d["architecture"] == "Mekusun" else zumizen_config(d, shapes)
         if d.get("architecture") == "Negunex":
             return negunex_config(d)
+        if d.get("architecture") == "Kakalorn":
+            return kakalorn_config(d)
         names = {f.name for f in dataclasses.fields(cls)}
         kw = {k: v for k, v in d.items() if k in names}
         if "num_experts" in d and "num_local_experts" not in d:
@@ -234,6 +238,36 @@ def zumizen_config(d: dict, shapes: Optional[dict] = None) -> ModelConfig:
         bos_token_id=d.get("bos", 0), eos_token_id=d.get("eos", -1), layer_specs=layers,
         embedding_scale=emb.get("scale", 1.0), bigram=emb.get("bigram"), logit_softcap=d.get("logit_softcap", 0.0),
         name=d.get("name", "zumizen"))
+
+
+KAKALORN_MIXERS = ("attention", "hgrn2", "latent_attention")
+
+
+def kakalorn_config(d: dict) -> ModelConfig:
+    """A Kakalorn ``config.json``: ``layers`` lists every layer (``type`` "attention", "hgrn2" or
+    "latent_attention", the ``mixer``'s sizes and constants, ``mlp`` or null), ``canon.taps`` the
+    taps of the short convolution in front of every mixer, ``norm.eps``, ``vocab``, ``width``. A
+    latent-attention layer with ``kv_from`` reads the cache of an earlier one, which must have a
+    down-projection of its own and the same latent size, rotated size and rotation."""
+    layers = [json.loads(json.dumps(l)) for l in d["layers"]]
+    for i, l in enumerate(layers):
+        if l["type"] not in KAKALORN_MIXERS:
+            raise ValueError(f"kakalorn: layer {i} has the unknown mixer type {l['type']!r}")
+        src = l["mixer"].get("kv_from") if l["type"] == "latent_attention" else None
+        if src is not None:
+            ok = 0 <= src < i and layers[src]["type"] == "latent_attention" and \
+                layers[src]["mixer"].get("kv_from") is None
+            if not ok or any(layers[src]["mixer"].get(k) != l["mixer"].get(k) for k in ("kv_rank", "rot_dim", "rot")):
+                raise ValueError(f"kakalorn: layer {i} cannot read the latent cache of layer {src}")
+    att = [l["mixer"] for l in layers if l["type"] == "attention"]
+    return ModelConfig(
+        model_type="kakalorn", hidden_size=d["width"], vocab_size=d["vocab"], num_hidden_layers=len(layers),
+        num_attention_heads=att[0]["heads"] if att else 1, num_key_value_heads=att[0]["kv_heads"] if att else 1,
+        head_dim=att[0]["dim"] if att else 1, v_head_dim=att[0]["dim"] if att else 0,
+        intermediate_size=max([l["mlp"]["ff"] for l in layers if l.get("mlp")] or [0]),
+        rms_norm_eps=d["norm"]["eps"], max_position_embeddings=d.get("max_position", 1 << 20),
+        bos_token_id=d.get("bos", 0), eos_token_id=d.get("eos", -1), layer_specs=layers,
+        conv_taps=int((d.get("canon") or {}).get("taps", 1)), name=d.get("name", "kakalorn"))
 
 
 def _llama(name, d, ffn, L, hq, hkv, vocab=128256, **kw):
@@ -414,6 +448,26 @@ def _tiny_zumizen() -> ModelConfig:
 
 
 _register(_tiny_zumizen())
+
+
+def _tiny_kakalorn() -> ModelConfig:
+    """Random-weight preset with one layer of every mixer kind and a layer that shares a latent cache."""
+    lat = {"heads": 4, "dim": 16, "rot_dim": 8, "vdim": 24, "kv_rank": 32, "q_rank": 48, "scale": 24 ** -0.5,
+           "rot": {"dims": 8, "base": 10000.0, "scaling": {"factor": 4.0, "original": 64, "fast": 8.0, "slow": 1.0}}}
+    att = {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 32, "scale": 32 ** -0.5,
+           "mask": {"size": 40, "keep_first": 3}, "rot": {"dims": 16, "base": 10000.0}}
+    rec = {"heads": 2, "dim": 16, "vdim": 32}
+    mlp = {"kind": "dense", "ff": 192}
+    return kakalorn_config({
+        "architecture": "Kakalorn", "name": "tiny-kakalorn", "width": 128, "vocab": 512, "norm": {"eps": 1e-6},
+        "canon": {"taps": 3}, "max_position": 4096, "eos": 1,
+        "layers": [{"type": "latent_attention", "mixer": lat, "mlp": mlp},
+                   {"type": "hgrn2", "mixer": rec, "mlp": mlp},
+                   {"type": "attention", "mixer": att, "mlp": None},
+                   {"type": "latent_attention", "mixer": dict(lat, kv_from=0), "mlp": mlp}]})
+
+
+_register(_tiny_kakalorn())
 
 
 def get_model_config(name_or_path: str) -> ModelConfig:

@@ -44,6 +44,10 @@ def model_class(cfg: ModelConfig):
         from .zumizen import ZumizenForCausalLM
 
         return ZumizenForCausalLM
+    if t == "kakalorn":
+        from .kakalorn import KakalornForCausalLM
+
+        return KakalornForCausalLM
     raise ValueError(f"unsupported model_type {t!r}")
 
 

@@ -20,6 +20,13 @@ constant is an argument, so another stack can reuse them.
 * ``ParallelMixer``    - two mixers that read the same input, their results added with two scales.
 * ``SigmoidMoE``       - gated experts chosen by sigmoid scores whose weight scales the expert's input.
 * ``BigramEmbedding``  - token embedding plus a hashed (previous, current) table.
+* ``GroupedAttention`` options for windowed stacks: values that are the projected keys, query / key
+  norms ahead of the rotation, a sliding window that keeps the sequence's first tokens, learned sinks.
+* ``LatentAttention`` options: queries through a normed latent of their own, interleaved rotary pairs,
+  ramp-scaled frequencies, one sigmoid gate per head, the cache of an earlier layer instead of its own.
+* ``Hgrn2Mixer``       - gated linear recurrence whose forget gate (bounded below) also sets what is written.
+* ``SquaredReluMLP``   - W_down relu(W_up h)^2.
+* ``InputConv``        - h + a short causal convolution of h, in front of a mixer.
 
 Recurrent state lives in the engine's state pool (engine/state_cache.py): a mixer with
 ``state_shapes()`` gets its per-slot tensors through ``bind_state``; the step's
@@ -54,39 +61,88 @@ def rope_table(dims: int, base: float, max_pos: int, device, scaling=None) -> to
 
     ``scaling`` = {factor, low, high, original}: frequency scaling by wavelength l = 2 pi / f -
     f stays where l < original / high, becomes f / factor where l > original / low, and between
-    the two is the blend (1 - s) f / factor + s f with s = (original / l - low) / (high - low)."""
+    the two is the blend (1 - s) f / factor + s f with s = (original / l - low) / (high - low).
+
+    ``scaling`` = {factor, original, fast, slow}: the ramp form. With n(t) = dims ln(original / (2 pi t))
+    / (2 ln base), the index at which a wave turns t times over ``original`` positions, lo =
+    max(floor(n(fast)), 0), hi = min(ceil(n(slow)), dims - 1) and r_i = clamp((i - lo) / max(hi - lo,
+    0.001), 0, 1) the frequency is (1 - r_i) f_i + r_i f_i / factor, and cos and sin are both
+    multiplied by 0.1 ln(factor) + 1."""
     half = dims // 2
     f = torch.tensor(base, dtype=torch.float64) ** (-2.0 * torch.arange(half, dtype=torch.float64) / dims)
-    if scaling:
+    mag = 1.0
+    if scaling and "fast" in scaling:
+        fac, orig = float(scaling["factor"]), float(scaling["original"])
+        turn = lambda t: dims * math.log(orig / (2.0 * math.pi * t)) / (2.0 * math.log(base))  # noqa: E731
+        lo = max(math.floor(turn(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(turn(float(scaling["slow"]))), dims - 1)
+        r = ((torch.arange(half, dtype=torch.float64) - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        f = f / fac * r + f * (1.0 - r)
+        mag = 0.1 * math.log(fac) + 1.0
+    elif scaling:
         fac, lo, hi, orig = (float(scaling[k]) for k in ("factor", "low", "high", "original"))
         wl = 2.0 * math.pi / f
         s = (orig / wl - lo) / (hi - lo)
         mid = (1.0 - s) * f / fac + s * f
         f = torch.where(wl < orig / hi, f, torch.where(wl > orig / lo, f / fac, mid))
     a = torch.arange(max_pos, dtype=torch.float64)[:, None] * f[None]
-    return torch.cat([a.cos(), a.sin()], -1).float().to(device)
+    return (torch.cat([a.cos(), a.sin()], -1) * mag).float().to(device)
 
 
 class LatentAttention(torch.nn.Module):
+    """Attention over a low-rank latent cache: the paged cache holds one row [normed latent | rotated
+    shared key part] per token; W_uk is absorbed into the query and W_uv applied to the latent read-out.
+
+    q_rank       > 0: queries go through a latent of their own, q = W_uq rms_norm(W_dq h) (weight
+                 ``dq_norm``); the layer's input projections [dq | dkv | gate] are then ONE product
+    interleaved  rotary pairs (2i, 2i+1) instead of (i, i + rot_dims/2)
+    rot_scaling  frequency scaling of ``rope_table``
+    gate         head h's result is multiplied by sigmoid(W_g h)_h, one number per head
+    kv_source    an earlier LatentAttention whose cache this layer reads instead of writing its own
+                 (no W_dkv here; W_uk, W_uv, queries and everything else are this layer's)
+    """
     is_latent = True
 
     def __init__(self, d_model, heads, dim, rot_dim, vdim, kv_rank, scale, rot_dims, rot_base, eps, max_pos,
-                 device, dtype):
+                 device, dtype, q_rank=0, interleaved=False, rot_scaling=None, gate=False, kv_source=None):
         super().__init__()
         if rot_dims > rot_dim or rot_dims % 2:
             raise ValueError(f"rotary dims {rot_dims} do not fit the rotated part {rot_dim}")
         self.H, self.dn, self.dr, self.dv, self.R = heads, dim, rot_dim, vdim, kv_rank
         self.scale, self.rot_dims, self.eps = float(scale), rot_dims, eps
-        self.q = ColumnLinear(d_model, heads * (dim + rot_dim), shard=False, device=device, dtype=dtype)
-        self.dkv = ColumnLinear(d_model, kv_rank + rot_dim, shard=False, device=device, dtype=dtype)
-        self.dkv_norm = _param((kv_rank,), device, dtype, fill=1.0)
+        self.q_rank, self.interleaved, self.has_gate = int(q_rank), bool(interleaved), bool(gate)
+        self._src = [kv_source] if kv_source is not None else None   # a list: not a submodule of this layer
+        if kv_source is not None and (kv_source.R, kv_source.dr, kv_source._src) != (kv_rank, rot_dim, None):
+            raise ValueError("a shared latent cache needs the same latent and rotated sizes and a layer that owns it")
+        self.fused = self.q_rank > 0 or self.has_gate
+        n_kv = 0 if kv_source is not None else kv_rank + rot_dim
+        if self.fused:
+            # one product of the layer input: [query latent (or queries) | latent + shared key | gate]
+            self.n_q = self.q_rank if self.q_rank else heads * (dim + rot_dim)
+            self.n_kv = n_kv
+            n = self.n_q + n_kv + (heads if gate else 0)
+            self.proj = ColumnLinear(d_model, -(-n // 8) * 8, shard=False, device=device, dtype=dtype)
+            if self.q_rank:
+                self.dq_norm = _param((self.q_rank,), device, dtype, fill=1.0)
+                self.uq = ColumnLinear(self.q_rank, heads * (dim + rot_dim), shard=False, device=device, dtype=dtype)
+        else:
+            self.q = ColumnLinear(d_model, heads * (dim + rot_dim), shard=False, device=device, dtype=dtype)
+            if kv_source is None:
+                self.dkv = ColumnLinear(d_model, kv_rank + rot_dim, shard=False, device=device, dtype=dtype)
+        if kv_source is None:
+            self.dkv_norm = _param((kv_rank,), device, dtype, fill=1.0)
         self.uk = _param((heads * dim, kv_rank), device, dtype)
         self.uv = _param((heads * vdim, kv_rank), device, dtype)
         self.o = ColumnLinear(heads * vdim, d_model, shard=False, device=device, dtype=dtype)
-        self.register_buffer("cos_sin", rope_table(rot_dims, rot_base, max_pos, device), persistent=False)
+        self.register_buffer("cos_sin", rope_table(rot_dims, rot_base, max_pos, device, rot_scaling),
+                             persistent=False)
         self.cache = None
         # what the runner's generic bookkeeping reads
         self.Hq, self.Hkv, self.D, self.window, self.sinks = heads, 1, kv_rank + rot_dim, 0, None
+
+    @property
+    def owns_cache(self) -> bool:
+        return self._src is None
 
     def kv_spec(self):
         return 1, 1, self.R + self.dr  # (planes, heads, dim): one latent row per token
@@ -98,16 +154,27 @@ class LatentAttention(torch.nn.Module):
     def forward(self, h, meta: AttnMeta):
         T, H, R, dn, dr = h.shape[0], self.H, self.R, self.dn, self.dr
         s = meta.seq
-        q = self.q(h)
-        kv = self.dkv(h)
+        gate = kv = None
+        if self.fused:
+            p = self.proj(h)
+            q = self.uq(sm.rms_norm(p[:, :self.q_rank], self.dq_norm, self.eps)) if self.q_rank else p[:, :self.n_q]
+            if self.n_kv:
+                kv = p[:, self.n_q:self.n_q + self.n_kv]
+            if self.has_gate:
+                gate = p[:, self.n_q + self.n_kv:self.n_q + self.n_kv + H]
+        else:
+            q = self.q(h)
+            if self._src is None:
+                kv = self.dkv(h)
+        cache = self.cache if self._src is None else self._src[0].cache
         q_abs = torch.empty(T, H, R + dr, dtype=h.dtype, device=h.device)
-        sm.latent_rope_cache(q, kv, self.dkv_norm, self.eps, meta.positions, self.cos_sin, H, dn, dr,
-                             self.rot_dims, R, meta.slot_mapping, self.cache, q_abs)
+        sm.latent_rope_cache(q, kv, self.dkv_norm if kv is not None else None, self.eps, meta.positions, self.cos_sin,
+                             H, dn, dr, self.rot_dims, R, meta.slot_mapping, cache, q_abs, self.interleaved)
         # absorb W_uk into the query: scores against the latent itself
         qn = q.view(T, H, dn + dr)[:, :, :dn].transpose(0, 1)                       # [H, T, dn]
         q_abs[:, :, :R].copy_(torch.bmm(qn, self.uk.view(H, dn, R)).transpose(0, 1))
-        o_lat = sm.latent_attention(q_abs, self.cache, s.tables, s.row_seq, s.row_len, self.scale, R,
-                                    rows_per_group=4 if s.max_q > 1 else 1, seq=s)
+        o_lat = sm.latent_attention(q_abs, cache, s.tables, s.row_seq, s.row_len, self.scale, R,
+                                    rows_per_group=4 if s.max_q > 1 else 1, seq=s, gate=gate)
         o = torch.bmm(o_lat.transpose(0, 1), self.uv.view(H, self.dv, R).transpose(1, 2))  # [H, T, dv]
         return self.o(o.transpose(0, 1).reshape(T, H * self.dv))
 
@@ -240,20 +307,33 @@ class GroupedAttention(torch.nn.Module):
     slopes       "pow2": the score of query i and key j loses 2^(-8 (h + 1) / heads) * (i - j)
     chunk        > 0: query i sees only keys j >= (i // chunk) * chunk (borders at multiples of chunk in the sequence's positions)
     sink         one more score of 0 per head in the softmax's denominator, without a value
+    sink         True: one more score of 0 per head in the softmax's denominator, without a value;
+                 "learned": that score is the parameter ``sink`` [heads] (it is not scaled)
     out_bias     the output projection has a bias
+    v_from_k     there is no value projection: the values are the projected keys (with their bias),
+                 before norm and rotation; needs vdim == dim
+    norm_first   the unit norms (and their weights) come before the rotation instead of after it
+    window       > 0: query i sees key j <= i only if i - j < window or j < keep_first; the kept first
+                 tokens keep their own positions
     """
     is_latent = False
 
     def __init__(self, d_model, heads, kv_heads, dim, vdim, scale, rot, eps, max_pos, device, dtype, bias=True,
                  interleaved=True, unit_norm=True, v_mix=False, gate=True, norm_weight=False, slopes=None, chunk=0,
-                 sink=False, out_bias=False):
+                 sink=False, out_bias=False, v_from_k=False, norm_first=False, window=0, keep_first=0):
         super().__init__()
         if heads % kv_heads:
             raise ValueError(f"{heads} query heads do not divide over {kv_heads} key/value heads")
+        if v_from_k and (vdim != dim or v_mix):
+            raise ValueError("values that are the keys need vdim == dim and no value mixing")
+        if window and chunk:
+            raise ValueError("a sliding window and chunks do not combine")
         self.Hq, self.Hkv, self.dim, self.vdim = heads, kv_heads, dim, vdim
         self.scale, self.eps, self.interleaved, self.unit_norm = float(scale), eps, interleaved, unit_norm
         self.v_mix, self.has_gate = bool(v_mix), bool(gate)
-        self.nq, self.nk, self.nv = heads * dim, kv_heads * dim, kv_heads * vdim
+        self.v_from_k, self.norm_first = bool(v_from_k), bool(norm_first)
+        self.win, self.keep_first = int(window), int(keep_first) if window else 0
+        self.nq, self.nk, self.nv = heads * dim, kv_heads * dim, 0 if v_from_k else kv_heads * vdim
         n = self.nq + self.nk + self.nv + (heads * vdim if gate else 0)
         self.n_out = -(-n // 8) * 8  # rows of 16-byte multiples for the vector loads downstream
         self.proj = ColumnLinear(d_model, self.n_out, shard=False, device=device, dtype=dtype)
@@ -274,6 +354,8 @@ class GroupedAttention(torch.nn.Module):
             self.slopes = torch.tensor([2.0 ** (-8.0 * (h + 1) / heads) for h in range(heads)], dtype=torch.float32,
                                        device=device)
         self.sink_logits = torch.zeros(heads, dtype=torch.float32, device=device) if sink else None
+        if sink == "learned":
+            self.sink = _param((heads,), device, dtype, fill=0.0)
         self.qk_w32 = None
         self.rot_dims = 0
         if rot:
@@ -294,6 +376,8 @@ class GroupedAttention(torch.nn.Module):
         self.lam = float(self.vmix.data.float().item())
         if self.norm_weight:
             self.qk_w32 = torch.stack([self.q_norm.data.float(), self.k_norm.data.float()]).contiguous()
+        if hasattr(self, "sink"):
+            self.sink_logits = self.sink.data.float()
 
     def kv_spec(self):
         return 1, self.Hkv, self.dim + self.vdim  # (planes, heads, row): [key | value] per kv head
@@ -318,11 +402,11 @@ class GroupedAttention(torch.nn.Module):
                 v_first = shared["v_first"] = torch.empty(T, self.nv, dtype=torch.float32, device=h.device)
         sm.qkv_rope_cache(p, self.bias32, meta.positions, self.cos_sin, self.Hq, self.Hkv, self.dim, self.vdim,
                           self.rot_dims, self.interleaved, self.eps if self.unit_norm else None, v_first, mode,
-                          self.lam, meta.slot_mapping, self.cache, q, self.qk_w32)
+                          self.lam, meta.slot_mapping, self.cache, q, self.qk_w32, self.norm_first, self.v_from_k)
         n0 = self.nq + self.nk + self.nv
         gate = p[:, n0:n0 + self.Hq * self.vdim] if self.has_gate else None
         o = sm.grouped_attention(q, self.cache, self.dim, self.vdim, self.scale, meta.seq, gate, self.slopes,
-                                 self.chunk, self.sink_logits)
+                                 self.chunk, self.sink_logits, self.win, self.keep_first)
         return self.o(o)
 
 
@@ -511,3 +595,73 @@ class BigramEmbedding(torch.nn.Module):
         """Fills the fp32 residual ``x`` [T, d]; returns it in the activation type."""
         return sm.bigram_embed(ids, self.table.weight, self.scale, self.bigram, self.buckets, self.mul_prev,
                                self.mul_cur, self.prev, meta.seq, x, out_dtype)
+
+
+class Hgrn2Mixer(torch.nn.Module):
+    """Gated linear recurrence per head whose forget gate also decides what is written. One
+    projection of the layer input gives [q | f | v]: q = silu(.) [heads, dim], v [heads, vdim] and the
+    gate f = lower + (1 - lower) sigmoid(. + f_bias) per head and channel, ``lower`` its bound from
+    below. Per head, in fp32:
+
+        S <- diag(f) S + (1 - f) v^T;  o = S^T q
+
+    then the head's RMS norm over vdim with ``norm`` [vdim] (shared by the heads) and the output
+    projection. State per sequence: S [heads, dim, vdim] fp32."""
+
+    def __init__(self, d_model, heads, dim, vdim, eps, device, dtype):
+        super().__init__()
+        self.H, self.dk, self.dv, self.eps = heads, dim, vdim, eps
+        self.nq, self.nv = heads * dim, heads * vdim
+        self.proj = ColumnLinear(d_model, -(-(2 * self.nq + self.nv) // 8) * 8, shard=False, device=device, dtype=dtype)
+        self.f_bias = _param((self.nq,), device, dtype, fill=0.0)
+        self.lower = _param((self.nq,), device, dtype, fill=0.0)
+        self.norm = _param((vdim,), device, dtype, fill=1.0)
+        self.o = ColumnLinear(self.nv, d_model, shard=False, device=device, dtype=dtype)
+        self.f_bias32 = self.lower32 = self.state = None
+
+    def finalize(self):
+        self.f_bias32, self.lower32 = self.f_bias.data.float(), self.lower.data.float()
+
+    def state_shapes(self):
+        return [((self.H, self.dk, self.dv), torch.float32)]
+
+    def bind_state(self, tensors):
+        (self.state,) = tensors
+
+    def forward(self, h, meta: AttnMeta):
+        y = sm.hgrn2_scan(self.proj(h), self.H, self.dk, self.dv, self.f_bias32, self.lower32, self.norm, self.eps,
+                          self.state, meta.seq)
+        return self.o(y)
+
+
+class SquaredReluMLP(torch.nn.Module):
+    """W_down relu(W_up h)^2."""
+
+    def __init__(self, d_model, ff, device, dtype):
+        super().__init__()
+        self.up = ColumnLinear(d_model, ff, shard=False, device=device, dtype=dtype)
+        self.down = ColumnLinear(ff, d_model, shard=False, device=device, dtype=dtype)
+
+    def forward(self, h):
+        return self.down(sm.relu2(self.up(h)))
+
+
+class InputConv(torch.nn.Module):
+    """h + conv(h): a causal convolution over time on each channel (``weight`` [channels, taps], the
+    last tap meets the current token, no bias, zeros before the sequence's start). State per
+    sequence: its last taps - 1 inputs."""
+
+    def __init__(self, channels, taps, device, dtype):
+        super().__init__()
+        self.C, self.taps, self.dtype = channels, int(taps), dtype
+        self.weight = _param((channels, self.taps), device, dtype, std=0.2)
+        self.state = None
+
+    def state_shapes(self):
+        return [((max(self.taps - 1, 1), self.C), self.dtype)]
+
+    def bind_state(self, tensors):
+        (self.state,) = tensors
+
+    def forward(self, h, meta: AttnMeta):
+        return sm.input_conv(h, self.weight, self.state, meta.seq)

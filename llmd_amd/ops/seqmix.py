@@ -4,7 +4,10 @@ scan, the generalized delta rule, zero-centred norms with layer scale, depth ave
 attention with its own key and value sizes (bias, rotary, unit norm, value mixing, gate), gated
 activations, score routing with a selection-only correction, gated experts with identity experts;
 the bigram embedding, the post-norm residual add, the gated delta rule, distance slopes / chunks /
-sinks in grouped attention, sigmoid routing with experts whose weight scales their input.
+sinks in grouped attention, sigmoid routing with experts whose weight scales their input; the embedding
+with the first norm, plain RMS norms of projections, the input convolution, the squared ReLU, the
+HGRN2 recurrence, sliding windows with kept first tokens, keys as values, per-head gates of latent
+attention.
 
 GPU tensors go to the ``llmd_amd._C_seqmix`` library (csrc/seqmix/*.hip, built on its own so a
 model that needs only these kernels compiles only these); it is templated on the activation
@@ -78,24 +81,28 @@ def depth_avg_norm(hist, n: int, coef, dst: int, norm_w, eps: float, out_dtype):
     return out
 
 
-def latent_rope_cache(q, kv, norm_w, eps, positions, cos_sin, H, dn, dr, rot_dims, R, slots, cache, q_abs):
+def latent_rope_cache(q, kv, norm_w, eps, positions, cos_sin, H, dn, dr, rot_dims, R, slots, cache, q_abs,
+                      interleaved: bool = False):
     """Rotate the rotary part of q into ``q_abs[..., R:]``; write [norm(kv[:, :R]) | rot(kv[:, R:])]
-    to the paged latent cache at ``slots`` (-1: no write). cos_sin [max_pos, rot_dims] fp32."""
+    to the paged latent cache at ``slots`` (-1: no write). cos_sin [max_pos, rot_dims] fp32; pairs
+    (i, i + rot_dims/2), or (2i, 2i+1) when ``interleaved``. ``kv`` None: a layer that reads another
+    layer's cache rotates its queries only."""
     if not q.is_cuda:
         return ref.latent_rope_cache(q, kv, norm_w, eps, positions, cos_sin, H, dn, dr, rot_dims, R, slots, cache,
-                                     q_abs)
+                                     q_abs, interleaved)
     native().latent_rope_cache(q, kv, norm_w, float(eps), positions, cos_sin, H, dn, dr, rot_dims, R, slots, cache,
-                               q_abs)
+                               q_abs, bool(interleaved))
 
 
 MFMA_ATTENTION = os.environ.get("LLMD_LATENT_MFMA", "1") == "1"
 
 
 def latent_attention(q_abs, cache, tables, row_seq, row_len, scale: float, R: int, rows_per_group: int = 1,
-                     seq=None):
+                     seq=None, gate=None):
     """Causal softmax attention of absorbed queries [T, H, R + dr] over the paged latent cache
     [blocks, bs, R + dr]; row t sees the first row_len[t] keys of sequence row_seq[t].
-    Returns the latent outputs [T, H, R].
+    Returns the latent outputs [T, H, R]. ``gate`` [T, H] (a column view of a projection): head h's
+    output is multiplied by sigmoid(gate[t, h]).
 
     bfloat16 with the step's ``seq`` description (engine/attn_meta.py SeqMeta): the matrix-core
     kernel over work items of up to 64 (token, head) rows of one sequence (R + dr <= 576, R <= 512,
@@ -104,7 +111,7 @@ def latent_attention(q_abs, cache, tables, row_seq, row_len, scale: float, R: in
     T, H, _ = q_abs.shape
     out = torch.empty(T, H, R, dtype=q_abs.dtype, device=q_abs.device)
     if not q_abs.is_cuda:
-        return ref.latent_attention(q_abs, cache, tables, row_seq, row_len, scale, R, out)
+        return ref.latent_attention(q_abs, cache, tables, row_seq, row_len, scale, R, out, gate)
     if MFMA_ATTENTION and seq is not None and q_abs.dtype == torch.bfloat16 and H <= 64:
         items = seq.attention_items(max(1, 64 // H))
         nsplit, split, po, pm = 1, 0, None, None
@@ -118,9 +125,9 @@ def latent_attention(q_abs, cache, tables, row_seq, row_len, scale: float, R: in
                 po = torch.empty(n * nsplit * 64 * R, dtype=torch.float32, device=q_abs.device)
                 pm = torch.empty(n * nsplit * 128, dtype=torch.float32, device=q_abs.device)
         if native().latent_attention_mfma(q_abs, cache, tables, items, row_len, float(scale), R, out, nsplit, split,
-                                          po, pm):
+                                          po, pm, gate):
             return out
-    native().latent_attention(q_abs, cache, tables, row_seq, row_len, float(scale), R, int(rows_per_group), out)
+    native().latent_attention(q_abs, cache, tables, row_seq, row_len, float(scale), R, int(rows_per_group), out, gate)
     return out
 
 
@@ -240,7 +247,7 @@ def hyper_update_norm(X, y, mix, w_out, next_in=None, next_w=None, eps: float = 
 
 # ---- grouped-query attention with its own key and value sizes
 def qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit_eps, v_first,
-                   v_mode, lam, slots, cache, q_out, qk_w=None):
+                   v_mode, lam, slots, cache, q_out, qk_w=None, norm_first: bool = False, v_from_k: bool = False):
     """From a fused projection [q | k | v | ...] of a step's tokens: add ``bias`` (fp32, over q|k|v),
     rotate the first ``rot_dims`` dimensions of every query and key head by the angles of ``cos_sin``
     [max_pos, rot_dims] = [cos | sin] (pairs (2i, 2i+1) when ``interleaved``, (i, i + rot_dims/2)
@@ -249,13 +256,16 @@ def qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, 
     [T, Hkv * vdim]; 2: v <- (1 - lam) v + lam v_first), write queries to ``q_out`` [T, Hq, dim] and
     the row [key | value] of every kv head to the paged ``cache`` [blocks, Hkv, bs, dim + vdim] at
     ``slots`` (-1: no write). ``qk_w`` fp32 [2, dim]: weights of the query and of the key norm (with
-    ``unit_eps``), shared by the heads. ``bias`` may be None. All arithmetic fp32."""
+    ``unit_eps``), shared by the heads. ``bias`` may be None. All arithmetic fp32.
+    ``norm_first``: the division by the root mean square and the weights come before the rotation.
+    ``v_from_k``: the projection is [q | k | ...] and the values are its keys (with their bias), as
+    projected - before norm and rotation (vdim == dim)."""
     if not qkv.is_cuda:
         return ref.qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit_eps,
-                                  v_first, v_mode, lam, slots, cache, q_out, qk_w)
+                                  v_first, v_mode, lam, slots, cache, q_out, qk_w, norm_first, v_from_k)
     native().qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, bool(interleaved),
                             unit_eps is not None, float(unit_eps or 0.0), v_first, int(v_mode), float(lam), slots, cache,
-                            q_out, qk_w)
+                            q_out, qk_w, bool(norm_first), bool(v_from_k))
 
 
 GQA_MFMA = os.environ.get("LLMD_GQA_MFMA", "1") == "1"
@@ -266,7 +276,8 @@ GQA_DECODE_WGS = int(os.environ.get("LLMD_GQA_DECODE_WGS", "2048"))  # workgroup
 GQA_RB2 = os.environ.get("LLMD_GQA_RB2", "0") == "1"
 
 
-def grouped_attention(q, cache, dim, vdim, scale: float, seq, gate=None, slopes=None, chunk: int = 0, sinks=None):
+def grouped_attention(q, cache, dim, vdim, scale: float, seq, gate=None, slopes=None, chunk: int = 0, sinks=None,
+                      window: int = 0, keep_first: int = 0):
     """Causal softmax attention of q [T, Hq, dim] over the paged cache [blocks, Hkv, bs, dim + vdim]
     (query head h reads kv head h // (Hq / Hkv)); row t sees the first seq.row_len[t] keys of its
     sequence. ``gate`` [T, Hq * vdim] (a column view of the fused projection): the result is
@@ -276,6 +287,8 @@ def grouped_attention(q, cache, dim, vdim, scale: float, seq, gate=None, slopes=
     ``chunk`` > 0: query i sees key j only inside its own chunk, j >= (i // chunk) * chunk; i and j are
     positions in the sequence, not in the step.
     ``sinks`` fp32 [Hq]: one more score per head in the softmax's denominator, without a value.
+    ``window`` > 0: query i sees key j <= i only if i - j < window or j < ``keep_first`` (positions in
+    the sequence); key tiles that lie between the kept first tokens and the window are not visited.
 
     bfloat16 runs on the matrix cores (work item = up to 64 (token, head-of-group) rows of one
     sequence and kv head); float32 and sizes outside the compiled forms on the fp32 FMA kernel."""
@@ -284,11 +297,17 @@ def grouped_attention(q, cache, dim, vdim, scale: float, seq, gate=None, slopes=
     out = torch.empty(T, Hq * vdim, dtype=q.dtype, device=q.device)
     if not q.is_cuda:
         return ref.grouped_attention(q, cache, dim, vdim, seq.tables, seq.row_seq, seq.row_len, scale, gate, out,
-                                     slopes, chunk, sinks)
+                                     slopes, chunk, sinks, window, keep_first)
     G = Hq // Hkv
-    chunk = int(chunk)
-    # keys a row can see at most: with chunks, its chunk (and the tile that the chunk starts in)
+    chunk, window = int(chunk), int(window)
+    keep_first = int(keep_first) if window else 0
+    if window and chunk:
+        raise ValueError("a sliding window and chunks do not combine")
+    # keys a row can see at most: with chunks, its chunk (and the tile that the chunk starts in); with a
+    # window, the tiles of the kept first tokens and those of the window
     span = min(seq.max_len, chunk + 32) if chunk else seq.max_len
+    if window:
+        span = min(seq.max_len, -(-keep_first // 32) * 32 + window + 32)
     if GQA_MFMA and q.dtype == torch.bfloat16 and G <= 64:
         rb = 2 if GQA_RB2 and seq.max_q * G > 64 else 1
         # workgroup ids run over the kv heads first: ids 256 apart (256 // Hkv items apart) share a CU
@@ -305,10 +324,10 @@ def grouped_attention(q, cache, dim, vdim, scale: float, seq, gate=None, slopes=
                 po = torch.empty(n * nsplit * 64 * vdim, dtype=torch.float32, device=q.device)
                 pm = torch.empty(n * nsplit * 128, dtype=torch.float32, device=q.device)
         if native().grouped_attention_mfma(q, cache, dim, vdim, seq.tables, items, seq.row_len, float(scale), gate,
-                                           out, nsplit, split, po, pm, rb, slopes, chunk, sinks):
+                                           out, nsplit, split, po, pm, rb, slopes, chunk, sinks, window, keep_first):
             return out
     native().grouped_attention(q, cache, dim, vdim, seq.tables, seq.row_seq, seq.row_len, float(scale), gate,
-                               4 if seq.max_q > 1 else 1, out, slopes, chunk, sinks)
+                               4 if seq.max_q > 1 else 1, out, slopes, chunk, sinks, window, keep_first)
     return out
 
 
@@ -427,4 +446,62 @@ def gated_delta_scan(xc, G: int, dk: int, H: int, dv: int, beta_raw, decay_raw, 
     native().gated_delta_scan(xc, int(G), int(dk), int(H), int(dv), beta_raw, decay_raw, A, dt_bias, gate_raw,
                               bool(gate_sigmoid), norm_w, float(eps), state, seq.seq_start, seq.seq_slot, seq.seq_init,
                               out)
+    return out
+
+
+# ---- embedding with the first norm, plain norms, input convolution, squared ReLU, HGRN2
+def embed_norm(ids, table, w, eps: float, x, out_dtype):
+    """x = table[ids] (the fp32 residual) and, from the same pass, rms_norm(x) * w in the activation type:
+    the first sublayer's input of a stack that norms before its sublayers."""
+    if not ids.is_cuda:
+        return ref.embed_norm(ids, table, w, eps, x, out_dtype)
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    native().embed_norm(ids, table, w, float(eps), x, out)
+    return out
+
+
+def rms_norm(y, w, eps: float):
+    """y / sqrt(mean(y^2) + eps) * w over the rows of y [T, n] (a column view of a projection is
+    fine), fp32 arithmetic, result in y's type."""
+    if not y.is_cuda:
+        return ref.rms_norm(y, w, eps)
+    out = torch.empty(y.shape, dtype=y.dtype, device=y.device)
+    native().rms_norm(y, w, float(eps), out)
+    return out
+
+
+def input_conv(h, w, state, seq):
+    """h + conv(h) per channel over each sequence's run: conv(h)_t = sum_j w[:, j] h_(t - taps + 1 + j),
+    continuing from the sequence's last taps - 1 inputs in ``state`` [slots, taps - 1, C] (read when
+    seq_init is set, zeros otherwise; rolled forward to the run's end)."""
+    out = torch.empty_like(h)
+    if not h.is_cuda:
+        return ref.input_conv(h, w, state, seq.seq_start, seq.seq_slot, seq.seq_init, out)
+    native().input_conv(h, w, state, seq.row_seq, seq.seq_start, seq.seq_slot, seq.seq_init, out)
+    return out
+
+
+def relu2(z):
+    """max(z, 0)^2."""
+    if not z.is_cuda:
+        return ref.relu2(z)
+    out = torch.empty_like(z)
+    native().relu2(z, out)
+    return out
+
+
+def hgrn2_scan(p, H: int, dk: int, dv: int, f_bias, lower, norm_w, eps: float, state, seq):
+    """HGRN2 over a step's runs. ``p`` [T, >= 2 H dk + H dv] = [q | f | v] as projected. Per token and
+    head, all fp32: q <- silu(q); f <- lower + (1 - lower) sigmoid(f + f_bias) (both fp32 [H dk]); then
+
+        S <- diag(f) S + (1 - f) v^T;  o = S^T q
+
+    (f scales the rows of S) and o / rms(o) * norm_w [dv]. ``state`` [slots, H, dk, dv] fp32 is
+    continued (seq_init) and written back. Returns [T, H dv]."""
+    out = torch.empty(p.shape[0], H * dv, dtype=p.dtype, device=p.device)
+    if not p.is_cuda:
+        return ref.hgrn2_scan(p, H, dk, dv, f_bias, lower, norm_w, eps, state, seq.seq_start, seq.seq_slot,
+                              seq.seq_init, out)
+    native().hgrn2_scan(p, int(H), int(dk), int(dv), f_bias, lower, norm_w, float(eps), state, seq.seq_start,
+                        seq.seq_slot, seq.seq_init, out)
     return out

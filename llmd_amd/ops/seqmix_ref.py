@@ -44,19 +44,32 @@ def _rot(v, cs, dims):
     return torch.cat([a * c - b * s, b * c + a * s, v[..., dims:].float()], -1)
 
 
-def latent_rope_cache(q, kv, norm_w, eps, positions, cos_sin, H, dn, dr, rot_dims, R, slots, cache, q_abs):
+def _rot_pairs(v, cs, dims):
+    """Pairs (2i, 2i+1) of the first ``dims`` entries."""
+    half = dims // 2
+    c, s = cs[..., :half], cs[..., half:]
+    a, b = v[..., 0:dims:2].float(), v[..., 1:dims:2].float()
+    r = torch.stack([a * c - b * s, b * c + a * s], -1).flatten(-2)
+    return torch.cat([r, v[..., dims:].float()], -1)
+
+
+def latent_rope_cache(q, kv, norm_w, eps, positions, cos_sin, H, dn, dr, rot_dims, R, slots, cache, q_abs,
+                      interleaved=False):
     T = q.shape[0]
+    rot = _rot_pairs if interleaved else _rot
     cs = cos_sin[positions]                                  # [T, rot_dims]
-    qr = _rot(q.view(T, H, dn + dr)[..., dn:], cs[:, None], rot_dims)
+    qr = rot(q.reshape(T, H, dn + dr)[..., dn:], cs[:, None], rot_dims)
     q_abs.view(T, H, R + dr)[..., R:] = qr.to(q_abs.dtype)
+    if kv is None:
+        return
     c = kv[:, :R].float()
     c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()
-    row = torch.cat([c, _rot(kv[:, R:], cs, rot_dims)], -1).to(cache.dtype)
+    row = torch.cat([c, rot(kv[:, R:], cs, rot_dims)], -1).to(cache.dtype)
     ok = slots >= 0
     cache.view(-1, R + dr)[slots[ok]] = row[ok]
 
 
-def latent_attention(q_abs, cache, tables, row_seq, row_len, scale, R, out):
+def latent_attention(q_abs, cache, tables, row_seq, row_len, scale, R, out, gate=None):
     T, H, Dk = q_abs.shape
     bs = cache.shape[1]
     flat = cache.view(-1, Dk)
@@ -67,7 +80,10 @@ def latent_attention(q_abs, cache, tables, row_seq, row_len, scale, R, out):
         K = flat[idx].float()                               # [n, Dk]
         s = (q_abs[t].float() @ K.T) * scale
         p = torch.softmax(s, -1)
-        out[t] = (p @ K[:, :R]).to(out.dtype)
+        o = p @ K[:, :R]
+        if gate is not None:
+            o = o * torch.sigmoid(gate[t].float())[:, None]
+        out[t] = o.to(out.dtype)
     return out
 
 
@@ -173,13 +189,24 @@ def hyper_update_norm(X, y, mix, w_out, next_in, next_w, eps, out_dtype):
 
 
 def qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit_eps, v_first,
-                   v_mode, lam, slots, cache, q_out, qk_w=None):
+                   v_mode, lam, slots, cache, q_out, qk_w=None, norm_first=False, v_from_k=False):
     T = qkv.shape[0]
-    nq, nk, nv = Hq * dim, Hkv * dim, Hkv * vdim
+    nq, nk, nv = Hq * dim, Hkv * dim, 0 if v_from_k else Hkv * vdim
     x = qkv[:, :nq + nk + nv].float()
     if bias is not None:
         x = x + bias.float()
-    q, k, v = x[:, :nq].view(T, Hq, dim), x[:, nq:nq + nk].view(T, Hkv, dim), x[:, nq + nk:].view(T, Hkv, vdim)
+    q, k = x[:, :nq].view(T, Hq, dim), x[:, nq:nq + nk].view(T, Hkv, dim)
+    v = k if v_from_k else x[:, nq + nk:].view(T, Hkv, vdim)
+
+    def unit(q, k):
+        q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + unit_eps)
+        k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + unit_eps)
+        if qk_w is not None:
+            q, k = q * qk_w[0].float(), k * qk_w[1].float()
+        return q, k
+
+    if unit_eps is not None and norm_first:
+        q, k = unit(q, k)
     if rot_dims:
         half = rot_dims // 2
         cs = cos_sin[positions]
@@ -195,11 +222,8 @@ def qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, 
             return torch.cat([r, t[..., rot_dims:]], -1)
 
         q, k = rot(q), rot(k)
-    if unit_eps is not None:
-        q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + unit_eps)
-        k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + unit_eps)
-        if qk_w is not None:
-            q, k = q * qk_w[0].float(), k * qk_w[1].float()
+    if unit_eps is not None and not norm_first:
+        q, k = unit(q, k)
     if v_mode == 1:
         v_first.copy_(v.reshape(T, nv))
     elif v_mode == 2:
@@ -223,7 +247,7 @@ def kv_views(cache, dim, vdim):
 
 
 def grouped_attention(q, cache, dim, vdim, tables, row_seq, row_len, scale, gate, out, slopes=None, chunk=0,
-                      sinks=None):
+                      sinks=None, window=0, keep_first=0):
     T, Hq, _ = q.shape
     nb, Hkv, bs, _ = cache.shape
     G = Hq // Hkv
@@ -233,6 +257,8 @@ def grouped_attention(q, cache, dim, vdim, tables, row_seq, row_len, scale, gate
         lo = ((n - 1) // chunk) * chunk if chunk else 0       # the first key of the query's chunk
         bt = tables[int(row_seq[t])].long()
         ar = torch.arange(lo, n)
+        if window:                                             # the kept first tokens and the window
+            ar = ar[(ar >= n - window) | (ar < keep_first)]
         K = kc[bt[ar // bs], :, ar % bs].float()              # [n - lo, Hkv, dim]
         V = vc[bt[ar // bs], :, :, ar % bs].float()           # [n - lo, Hkv, vdim]
         qt = q[t].float().view(Hkv, G, dim)
@@ -241,7 +267,7 @@ def grouped_attention(q, cache, dim, vdim, tables, row_seq, row_len, scale, gate
             s = s - slopes.float().view(Hkv, G, 1) * (n - 1 - ar).float()
         if sinks is not None:                                   # one more score per head, without a value
             s = torch.cat([s, sinks.float().view(Hkv, G, 1)], -1)
-        p = torch.softmax(s, -1)[..., :n - lo]
+        p = torch.softmax(s, -1)[..., :ar.numel()]
         o = torch.einsum("hgn,nhv->hgv", p, V).reshape(Hq * vdim)
         if gate is not None:
             o = o * torch.sigmoid(gate[t].float())
@@ -353,4 +379,58 @@ def gated_delta_scan(xc, G, dk, H, dv, beta_raw, decay_raw, A, dt_bias, gate_raw
         if hi > lo:
             state[sl] = S
     del per_channel
+    return out
+
+
+# ---- embedding with the first norm, plain norms, input convolution, squared ReLU, HGRN2
+def embed_norm(ids, table, w, eps, x, out_dtype):
+    x.copy_(table[ids].float())
+    return (_rms(x, eps) * w.float()).to(out_dtype)
+
+
+def rms_norm(y, w, eps):
+    return (_rms(y.float(), eps) * w.float()).to(y.dtype)
+
+
+def input_conv(h, w, state, seq_start, seq_slot, seq_init, out):
+    C, taps = w.shape
+    wf = w.float()
+    for i in range(seq_slot.numel()):
+        lo, hi, sl = int(seq_start[i]), int(seq_start[i + 1]), int(seq_slot[i])
+        if hi == lo:
+            continue
+        x = h[lo:hi].float()
+        prev = state[sl, :taps - 1].float() if int(seq_init[i]) else torch.zeros(taps - 1, C)
+        xp = torch.cat([prev, x])
+        acc = x.clone()
+        for j in range(taps):
+            acc += xp[j:j + hi - lo] * wf[:, j]
+        out[lo:hi] = acc.to(out.dtype)
+        if taps > 1:
+            state[sl, :taps - 1] = xp[-(taps - 1):].to(state.dtype)
+    return out
+
+
+def relu2(z):
+    a = torch.relu(z.float())
+    return (a * a).to(z.dtype)
+
+
+def hgrn2_scan(p, H, dk, dv, f_bias, lower, norm_w, eps, state, seq_start, seq_slot, seq_init, out):
+    T = p.shape[0]
+    nq = H * dk
+    q = F.silu(p[:, :nq].float()).view(T, H, dk)
+    low = lower.float()
+    f = (low + (1.0 - low) * torch.sigmoid(p[:, nq:2 * nq].float() + f_bias.float())).view(T, H, dk)
+    v = p[:, 2 * nq:2 * nq + H * dv].float().view(T, H, dv)
+    for i in range(seq_slot.numel()):
+        lo, hi, sl = int(seq_start[i]), int(seq_start[i + 1]), int(seq_slot[i])
+        if hi == lo:
+            continue
+        S = state[sl].clone() if int(seq_init[i]) else torch.zeros_like(state[sl])
+        for t in range(lo, hi):
+            S = f[t][:, :, None] * S + (1.0 - f[t])[:, :, None] * v[t][:, None]
+            o = torch.einsum("hkv,hk->hv", S, q[t])
+            out[t] = (_rms(o, eps) * norm_w.float()).reshape(H * dv).to(out.dtype)
+        state[sl] = S
     return out
