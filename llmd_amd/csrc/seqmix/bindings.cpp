@@ -16,11 +16,19 @@ void sm_depth_avg_norm(float*, int64_t, int, const float*, int, const void*, flo
 void sm_xielu(const void*, float, float, void*, int64_t, int, hipStream_t);
 void sm_softcap(float*, float, int64_t, hipStream_t);
 void sm_latent_rope_cache(const void*, int64_t, const void*, int64_t, const void*, float, const int64_t*, const float*,
-                          int, int, int, int, int, const int64_t*, void*, void*, int, int, hipStream_t);
+                          int, int, int, int, int, const int64_t*, void*, void*, int, int, int, hipStream_t);
 int sm_latent_attention(const void*, const void*, const int*, int, int, const int*, const int*, float, int, int, int,
-                        int, int, void*, int, hipStream_t);
+                        int, int, void*, int, const void*, int64_t, hipStream_t);
 int sm_latent_attention_mfma(const void*, const void*, const int*, int, int, const int*, int, const int*, float, int,
-                             int, int, void*, int, int, float*, float*, hipStream_t);
+                             int, int, void*, int, int, float*, float*, const void*, int64_t, hipStream_t);
+void sm_embed_norm(const int64_t*, const void*, int64_t, const void*, float, float*, void*, int, int, int, hipStream_t);
+void sm_rms_norm_rows(const void*, int64_t, const void*, float, void*, int, int, int, hipStream_t);
+void sm_relu2(const void*, void*, int64_t, int, hipStream_t);
+void sm_input_conv(const void*, int, const void*, int, void*, const int*, const int*, const int*, const int*, void*,
+                   int, int, int, hipStream_t);
+int sm_hgrn2_scan(const void*, int64_t, int, int, int, const float*, const float*, const void*, float, float*,
+                  const int*, const int*, const int*, void*, float*, float*, float*, float*, int, int, int,
+                  hipStream_t);
 void sm_causal_conv_silu(const void*, int64_t, int, const void*, const void*, int, void*, const int*, const int*,
                          const int*, void*, int, int, int, hipStream_t);
 int sm_selective_scan(const void*, const void*, const void*, const float*, const void*, int64_t, int, int, const void*,
@@ -34,13 +42,14 @@ void sm_hyper_update_norm(float*, const void*, int64_t, const float*, const floa
                           void*, int, int, int, int, hipStream_t);
 void sm_gated_act(const void*, int64_t, int, int, void*, int, int, hipStream_t);
 void sm_qkv_rope_cache(const void*, int64_t, const float*, const int64_t*, const float*, int, int, int, int, int, int,
-                       int, float, float*, int, float, const int64_t*, void*, int, void*, const float*, int, int,
-                       hipStream_t);
+                       int, float, float*, int, float, const int64_t*, void*, int, void*, const float*, int, int, int,
+                       int, hipStream_t);
 int sm_grouped_attention(const void*, const void*, const int*, int, int, const int*, const int*, float, int, int, int,
-                         int, int, int, const void*, int64_t, void*, int, const float*, int, const float*, hipStream_t);
+                         int, int, int, const void*, int64_t, void*, int, const float*, int, const float*, int, int,
+                         hipStream_t);
 int sm_grouped_attention_mfma(const void*, const void*, const int*, int, int, const int*, int, const int*, float, int,
                               int, int, int, const void*, int64_t, void*, int, int, float*, float*, int, const float*,
-                              int, const float*, hipStream_t);
+                              int, const float*, int, int, hipStream_t);
 void sm_moe_route_scores(const float*, const float*, int, int, int*, float*, int, hipStream_t);
 void sm_moe_route(const float*, int, int, int*, float*, int, int, hipStream_t);
 void sm_moe_group(const int*, int, int, int*, int*, int*, int, hipStream_t);
@@ -158,15 +167,20 @@ void softcap(Tensor x, double cap) {
   sm_softcap(x.data_ptr<float>(), (float)cap, x.numel(), cur());
 }
 
-void latent_rope_cache(Tensor q, Tensor kv, Tensor norm_w, double eps, Tensor positions, Tensor cos_sin, int64_t H,
-                       int64_t dn, int64_t dr, int64_t rot_dims, int64_t R, Tensor slots, Tensor cache, Tensor q_abs) {
+void latent_rope_cache(Tensor q, std::optional<Tensor> kv_, std::optional<Tensor> norm_w_, double eps, Tensor positions,
+                       Tensor cos_sin, int64_t H, int64_t dn, int64_t dr, int64_t rot_dims, int64_t R, Tensor slots,
+                       Tensor cache, Tensor q_abs, bool interleaved) {
   const c10::hip::OptionalHIPGuard g(dev_of(q));
   TORCH_CHECK(q.is_cuda() && act_ok(q) && q.dim() == 2 && q.stride(1) == 1 && q.size(1) == H * (dn + dr), "q");
   const int T = q.size(0);
-  CHECK_ACT(kv, q);
-  TORCH_CHECK(kv.dim() == 2 && kv.stride(1) == 1 && kv.size(0) == T && kv.size(1) == R + dr, "kv");
-  CHECK_ACT(norm_w, q);
-  TORCH_CHECK(norm_w.is_contiguous() && norm_w.numel() == R, "latent norm weight");
+  TORCH_CHECK(kv_.has_value() == norm_w_.has_value(), "kv and its norm weight come together");
+  if (kv_) {
+    const Tensor &kv = *kv_, &norm_w = *norm_w_;
+    CHECK_ACT(kv, q);
+    TORCH_CHECK(kv.dim() == 2 && kv.stride(1) == 1 && kv.size(0) == T && kv.size(1) == R + dr, "kv");
+    CHECK_ACT(norm_w, q);
+    TORCH_CHECK(norm_w.is_contiguous() && norm_w.numel() == R, "latent norm weight");
+  }
   TORCH_CHECK(positions.is_cuda() && positions.scalar_type() == torch::kInt64 && positions.is_contiguous() &&
                   positions.numel() == T, "positions");
   TORCH_CHECK(slots.is_cuda() && slots.scalar_type() == torch::kInt64 && slots.is_contiguous() && slots.numel() == T,
@@ -178,13 +192,21 @@ void latent_rope_cache(Tensor q, Tensor kv, Tensor norm_w, double eps, Tensor po
   CHECK_ACT(q_abs, q);
   TORCH_CHECK(q_abs.is_contiguous() && q_abs.numel() == (int64_t)T * H * (R + dr), "q_abs");
   // positions and slots are produced by the runner within [0, max_pos) and the pool
-  sm_latent_rope_cache(q.data_ptr(), q.stride(0), kv.data_ptr(), kv.stride(0), norm_w.data_ptr(), (float)eps,
-                       positions.data_ptr<int64_t>(), cos_sin.data_ptr<float>(), H, dn, dr, rot_dims, R,
-                       slots.data_ptr<int64_t>(), cache.data_ptr(), q_abs.data_ptr(), T, is_f32(q), cur());
+  sm_latent_rope_cache(q.data_ptr(), q.stride(0), kv_ ? kv_->data_ptr() : nullptr, kv_ ? kv_->stride(0) : 0,
+                       norm_w_ ? norm_w_->data_ptr() : nullptr, (float)eps, positions.data_ptr<int64_t>(),
+                       cos_sin.data_ptr<float>(), H, dn, dr, rot_dims, R, slots.data_ptr<int64_t>(), cache.data_ptr(),
+                       q_abs.data_ptr(), interleaved ? 1 : 0, T, is_f32(q), cur());
+}
+
+void check_head_gate(const std::optional<Tensor>& gate, const Tensor& q_abs) {
+  if (!gate) return;
+  CHECK_ACT(*gate, q_abs);
+  TORCH_CHECK(gate->dim() == 2 && gate->size(0) == q_abs.size(0) && gate->size(1) == q_abs.size(1) &&
+                  gate->stride(1) == 1, "gate [T, H]");
 }
 
 void latent_attention(Tensor q_abs, Tensor cache, Tensor tables, Tensor row_seq, Tensor row_len, double scale,
-                      int64_t R, int64_t qt, Tensor out) {
+                      int64_t R, int64_t qt, Tensor out, std::optional<Tensor> gate) {
   const c10::hip::OptionalHIPGuard g(dev_of(q_abs));
   TORCH_CHECK(q_abs.is_cuda() && act_ok(q_abs) && q_abs.dim() == 3 && q_abs.is_contiguous(), "q_abs [T, H, Dk]");
   const int T = q_abs.size(0), H = q_abs.size(1), Dk = q_abs.size(2);
@@ -197,15 +219,17 @@ void latent_attention(Tensor q_abs, Tensor cache, Tensor tables, Tensor row_seq,
   CHECK_ACT(out, q_abs);
   TORCH_CHECK(out.is_contiguous() && out.numel() == (int64_t)T * H * R, "out [T, H, R]");
   TORCH_CHECK(qt == 1 || qt == 4, "rows per workgroup: 1 or 4");
+  check_head_gate(gate, q_abs);
   const int rc = sm_latent_attention(q_abs.data_ptr(), cache.data_ptr(), tables.data_ptr<int>(), tables.size(1),
                                      cache.size(1), row_seq.data_ptr<int>(), row_len.data_ptr<int>(), (float)scale, H,
-                                     R, Dk, T, qt, out.data_ptr(), is_f32(q_abs), cur());
+                                     R, Dk, T, qt, out.data_ptr(), is_f32(q_abs), gate ? gate->data_ptr() : nullptr,
+                                     gate ? gate->stride(0) : 0, cur());
   TORCH_CHECK(rc == 0, "latent_attention: latent rank above 1024 or rows too wide for the LDS tile");
 }
 
 bool latent_attention_mfma(Tensor q_abs, Tensor cache, Tensor tables, Tensor items, Tensor row_len, double scale,
                            int64_t R, Tensor out, int64_t nsplit, int64_t split_keys, c10::optional<Tensor> part_o,
-                           c10::optional<Tensor> part_ml) {
+                           c10::optional<Tensor> part_ml, std::optional<Tensor> gate) {
   const c10::hip::OptionalHIPGuard g(dev_of(q_abs));
   TORCH_CHECK(q_abs.is_cuda() && q_abs.scalar_type() == torch::kBFloat16 && q_abs.dim() == 3 && q_abs.is_contiguous(),
               "q_abs [T, H, Dk] bf16");
@@ -221,6 +245,7 @@ bool latent_attention_mfma(Tensor q_abs, Tensor cache, Tensor tables, Tensor ite
   // the items are built by ops.seqmix.attention_items from the step's run lengths: rows inside [0, T),
   // tokens * H <= 64
   float *po = nullptr, *pm = nullptr;
+  check_head_gate(gate, q_abs);
   TORCH_CHECK(nsplit >= 1 && nsplit <= 1024, "key ranges per item");
   if (nsplit > 1) {
     TORCH_CHECK(split_keys >= 32 && split_keys % 32 == 0, "keys per range: a multiple of 32");
@@ -234,7 +259,8 @@ bool latent_attention_mfma(Tensor q_abs, Tensor cache, Tensor tables, Tensor ite
   }
   return sm_latent_attention_mfma(q_abs.data_ptr(), cache.data_ptr(), tables.data_ptr<int>(), tables.size(1),
                                   cache.size(1), items.data_ptr<int>(), items.size(0), row_len.data_ptr<int>(),
-                                  (float)scale, H, R, Dk, out.data_ptr(), nsplit, split_keys, po, pm, cur()) == 0;
+                                  (float)scale, H, R, Dk, out.data_ptr(), nsplit, split_keys, po, pm,
+                                  gate ? gate->data_ptr() : nullptr, gate ? gate->stride(0) : 0, cur()) == 0;
 }
 
 void causal_conv_silu(Tensor xz, int64_t C, Tensor w, Tensor b, Tensor state, Tensor seq_start, Tensor seq_slot,
@@ -377,10 +403,11 @@ void gated_act(Tensor gu, int64_t F, int64_t kind, Tensor out) {
 void qkv_rope_cache(Tensor qkv, std::optional<Tensor> bias, Tensor positions, std::optional<Tensor> cos_sin, int64_t Hq,
                     int64_t Hkv, int64_t dim, int64_t vdim, int64_t rot_dims, bool interleaved, bool unit, double eps,
                     std::optional<Tensor> v_first, int64_t v_mode, double lam, Tensor slots, Tensor cache,
-                    Tensor q_out, std::optional<Tensor> qk_w) {
+                    Tensor q_out, std::optional<Tensor> qk_w, bool norm_first, bool v_from_k) {
   const c10::hip::OptionalHIPGuard g(dev_of(qkv));
   TORCH_CHECK(qkv.is_cuda() && act_ok(qkv) && qkv.dim() == 2 && qkv.stride(1) == 1, "qkv");
-  const int64_t T = qkv.size(0), n = (Hq + Hkv) * dim + Hkv * vdim;
+  TORCH_CHECK(!v_from_k || (vdim == dim && v_mode == 0), "keys as values: vdim == dim, no value mixing");
+  const int64_t T = qkv.size(0), n = (Hq + Hkv) * dim + (v_from_k ? 0 : Hkv * vdim);
   TORCH_CHECK(Hq >= 1 && Hkv >= 1 && Hq % Hkv == 0 && dim >= 1 && dim <= 512 && vdim >= 1 && qkv.size(1) >= n, "sizes");
   TORCH_CHECK(rot_dims >= 0 && rot_dims <= dim && rot_dims % 2 == 0, "rotary dims");
   TORCH_CHECK(positions.is_cuda() && positions.scalar_type() == torch::kInt64 && positions.is_contiguous() &&
@@ -414,7 +441,8 @@ void qkv_rope_cache(Tensor qkv, std::optional<Tensor> bias, Tensor positions, st
                     positions.data_ptr<int64_t>(), rot_dims ? cos_sin->data_ptr<float>() : nullptr, Hq, Hkv, dim, vdim,
                     rot_dims, interleaved ? 1 : 0, unit ? 1 : 0, (float)eps, v_mode ? v_first->data_ptr<float>() : nullptr,
                     v_mode, (float)lam, slots.data_ptr<int64_t>(), cache.data_ptr(), cache.size(2), q_out.data_ptr(),
-                    qk_w ? qk_w->data_ptr<float>() : nullptr, T, is_f32(qkv), cur());
+                    qk_w ? qk_w->data_ptr<float>() : nullptr, norm_first ? 1 : 0, v_from_k ? 1 : 0, T, is_f32(qkv),
+                    cur());
 }
 
 void check_gqa(const Tensor& q, const Tensor& cache, int64_t dim, int64_t vdim, const Tensor& tables,
@@ -442,11 +470,18 @@ void check_gqa(const Tensor& q, const Tensor& cache, int64_t dim, int64_t vdim, 
   }
 }
 
+void check_window(int64_t window, int64_t keep, int64_t chunk) {
+  TORCH_CHECK(window >= 0 && window < (1ll << 30) && keep >= 0 && keep < (1ll << 30) && (window == 0 || chunk == 0),
+              "window / kept first tokens (not with chunks)");
+}
+
 void grouped_attention(Tensor q, Tensor cache, int64_t dim, int64_t vdim, Tensor tables, Tensor row_seq, Tensor row_len,
                        double scale, std::optional<Tensor> gate, int64_t rows_per_group, Tensor out,
-                       std::optional<Tensor> slopes, int64_t chunk, std::optional<Tensor> sinks) {
+                       std::optional<Tensor> slopes, int64_t chunk, std::optional<Tensor> sinks, int64_t window,
+                       int64_t keep) {
   const c10::hip::OptionalHIPGuard g(dev_of(q));
   check_gqa(q, cache, dim, vdim, tables, row_len, gate, out, slopes, chunk, sinks);
+  check_window(window, keep, chunk);
   CHECK_I32(row_seq);
   TORCH_CHECK(row_seq.numel() == q.size(0) && (rows_per_group == 1 || rows_per_group == 4), "row_seq [T]");
   const int rc = sm_grouped_attention(q.data_ptr(), cache.data_ptr(), tables.data_ptr<int>(), tables.size(1),
@@ -454,16 +489,18 @@ void grouped_attention(Tensor q, Tensor cache, int64_t dim, int64_t vdim, Tensor
                                       q.size(1), cache.size(1), dim, vdim, q.size(0), rows_per_group,
                                       gate ? gate->data_ptr() : nullptr, gate ? gate->stride(0) : 0, out.data_ptr(),
                                       is_f32(q), slopes ? slopes->data_ptr<float>() : nullptr, chunk,
-                                      sinks ? sinks->data_ptr<float>() : nullptr, cur());
+                                      sinks ? sinks->data_ptr<float>() : nullptr, window, keep, cur());
   TORCH_CHECK(rc == 0, "grouped_attention: head sizes too large for the kernel (vdim <= 1024, one key tile in LDS)");
 }
 
 bool grouped_attention_mfma(Tensor q, Tensor cache, int64_t dim, int64_t vdim, Tensor tables, Tensor items,
                             Tensor row_len, double scale, std::optional<Tensor> gate, Tensor out, int64_t nsplit,
                             int64_t split_keys, std::optional<Tensor> part_o, std::optional<Tensor> part_ml,
-                            int64_t rb, std::optional<Tensor> slopes, int64_t chunk, std::optional<Tensor> sinks) {
+                            int64_t rb, std::optional<Tensor> slopes, int64_t chunk, std::optional<Tensor> sinks,
+                            int64_t window, int64_t keep) {
   const c10::hip::OptionalHIPGuard g(dev_of(q));
   check_gqa(q, cache, dim, vdim, tables, row_len, gate, out, slopes, chunk, sinks);
+  check_window(window, keep, chunk);
   TORCH_CHECK(q.scalar_type() == torch::kBFloat16, "bf16 only");
   CHECK_I32(items);
   TORCH_CHECK(items.dim() == 2 && items.size(1) == 3, "items [n, 3]");
@@ -484,7 +521,7 @@ bool grouped_attention_mfma(Tensor q, Tensor cache, int64_t dim, int64_t vdim, T
                                            (float)scale, q.size(1), Hkv, dim, vdim, gate ? gate->data_ptr() : nullptr,
                                            gate ? gate->stride(0) : 0, out.data_ptr(), nsplit, split_keys, po, pm,
                                            rb, slopes ? slopes->data_ptr<float>() : nullptr, chunk,
-                                           sinks ? sinks->data_ptr<float>() : nullptr, cur());
+                                           sinks ? sinks->data_ptr<float>() : nullptr, window, keep, cur());
   return rc == 0;
 }
 
@@ -672,6 +709,92 @@ void gated_delta_scan(Tensor xc, int64_t G, int64_t dk, int64_t H, int64_t dv, T
   TORCH_CHECK(rc == 0, "gated_delta_scan: key size above 256");
 }
 
+void embed_norm(Tensor ids, Tensor table, Tensor w, double eps, Tensor x, Tensor out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(x));
+  TORCH_CHECK(ids.is_cuda() && ids.scalar_type() == torch::kInt64 && ids.is_contiguous() && ids.dim() == 1, "ids");
+  TORCH_CHECK(table.is_cuda() && act_ok(table) && table.dim() == 2 && table.is_contiguous(), "table");
+  const int64_t T = ids.numel(), d = table.size(1);
+  CHECK_ACT(w, table);
+  CHECK_ACT(out, table);
+  CHECK_F32(x);
+  TORCH_CHECK(w.is_contiguous() && w.numel() == d && x.numel() == T * d && out.is_contiguous() && out.numel() == T * d,
+              "w [d], x / out [T, d]");
+  sm_embed_norm(ids.data_ptr<int64_t>(), table.data_ptr(), table.size(0), w.data_ptr(), (float)eps,
+                x.data_ptr<float>(), out.data_ptr(), T, d, is_f32(table), cur());
+}
+
+void rms_norm(Tensor y, Tensor w, double eps, Tensor out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(y));
+  TORCH_CHECK(y.is_cuda() && act_ok(y) && y.dim() == 2 && y.stride(1) == 1, "y [T, n] rows");
+  CHECK_ACT(w, y);
+  CHECK_ACT(out, y);
+  TORCH_CHECK(w.is_contiguous() && w.numel() == y.size(1) && out.is_contiguous() && out.numel() == y.numel(),
+              "w [n], out [T, n]");
+  sm_rms_norm_rows(y.data_ptr(), y.stride(0), w.data_ptr(), (float)eps, out.data_ptr(), y.size(0), y.size(1),
+                   is_f32(y), cur());
+}
+
+void relu2(Tensor z, Tensor out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(z));
+  TORCH_CHECK(z.is_cuda() && act_ok(z) && z.is_contiguous(), "z");
+  CHECK_ACT(out, z);
+  TORCH_CHECK(out.is_contiguous() && out.numel() == z.numel(), "out");
+  sm_relu2(z.data_ptr(), out.data_ptr(), z.numel(), is_f32(z), cur());
+}
+
+void input_conv(Tensor h, Tensor w, Tensor state, Tensor row_seq, Tensor seq_start, Tensor seq_slot, Tensor seq_init,
+                Tensor out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(h));
+  TORCH_CHECK(h.is_cuda() && act_ok(h) && h.dim() == 2 && h.is_contiguous(), "h [T, C]");
+  const int64_t T = h.size(0), C = h.size(1);
+  CHECK_ACT(w, h);
+  CHECK_ACT(state, h);
+  CHECK_ACT(out, h);
+  TORCH_CHECK(w.dim() == 2 && w.is_contiguous() && w.size(0) == C && w.size(1) >= 1, "conv weights [C, taps]");
+  const int taps = w.size(1);
+  TORCH_CHECK(state.dim() == 3 && state.is_contiguous() && state.size(2) == C &&
+                  (taps == 1 || state.size(1) == taps - 1), "conv state [slots, taps-1, C]");
+  check_seq(seq_start, seq_slot, seq_init, state.size(0));
+  CHECK_I32(row_seq);
+  TORCH_CHECK(row_seq.numel() == T && seq_slot.numel() <= 65535, "row_seq [T]");
+  TORCH_CHECK(out.is_contiguous() && out.numel() == T * C, "out [T, C]");
+  sm_input_conv(h.data_ptr(), C, w.data_ptr(), taps, state.data_ptr(), row_seq.data_ptr<int>(),
+                seq_start.data_ptr<int>(), seq_slot.data_ptr<int>(), seq_init.data_ptr<int>(), out.data_ptr(), T,
+                seq_slot.numel(), is_f32(h), cur());
+}
+
+void hgrn2_scan(Tensor p, int64_t H, int64_t dk, int64_t dv, Tensor f_bias, Tensor lower, Tensor norm_w, double eps,
+                Tensor state, Tensor seq_start, Tensor seq_slot, Tensor seq_init, Tensor out) {
+  const c10::hip::OptionalHIPGuard g(dev_of(p));
+  TORCH_CHECK(H >= 1 && dk >= 1 && dv >= 1, "head count and sizes");
+  TORCH_CHECK(p.is_cuda() && act_ok(p) && p.dim() == 2 && p.stride(1) == 1 && p.size(1) >= 2 * H * dk + H * dv,
+              "p [T, q | f | v]");
+  const int64_t T = p.size(0);
+  CHECK_ACT(norm_w, p);
+  CHECK_ACT(out, p);
+  CHECK_F32(f_bias);
+  CHECK_F32(lower);
+  CHECK_F32(state);
+  TORCH_CHECK(f_bias.numel() == H * dk && lower.numel() == H * dk && norm_w.is_contiguous() && norm_w.numel() == dv,
+              "f_bias, lower [H dk], norm_w [dv]");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == dk && state.size(3) == dv,
+              "state [slots, H, dk, dv]");
+  check_seq(seq_start, seq_slot, seq_init, state.size(0));
+  TORCH_CHECK(out.is_contiguous() && out.dim() == 2 && out.size(0) == T && out.size(1) == H * dv, "out [T, H dv]");
+  const int64_t KD = sm_gated_delta_rows(dk);
+  TORCH_CHECK(KD > 0, "hgrn2_scan: key size above 256");
+  TORCH_CHECK(seq_slot.numel() <= 65535, "too many sequences in a step");
+  // fp32 workspaces of the three kernels: [qn | kn | dec | o_raw]
+  const int64_t n_qk = T * H * KD, n_o = T * H * dv;
+  Tensor ws = torch::empty({3 * n_qk + n_o + 4}, torch::dtype(torch::kFloat32).device(p.device()));
+  float* w0 = ws.data_ptr<float>();
+  const int rc = sm_hgrn2_scan(p.data_ptr(), p.stride(0), H, dk, dv, f_bias.data_ptr<float>(), lower.data_ptr<float>(),
+                               norm_w.data_ptr(), (float)eps, state.data_ptr<float>(), seq_start.data_ptr<int>(),
+                               seq_slot.data_ptr<int>(), seq_init.data_ptr<int>(), out.data_ptr(), w0, w0 + n_qk,
+                               w0 + 2 * n_qk, w0 + 3 * n_qk, T, seq_slot.numel(), is_f32(p), cur());
+  TORCH_CHECK(rc == 0, "hgrn2_scan: key size above 256");
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -702,4 +825,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("bigram_embed", &bigram_embed);
   m.def("post_norm_add", &post_norm_add);
   m.def("gated_delta_scan", &gated_delta_scan);
+  m.def("embed_norm", &embed_norm);
+  m.def("rms_norm", &rms_norm);
+  m.def("relu2", &relu2);
+  m.def("input_conv", &input_conv);
+  m.def("hgrn2_scan", &hgrn2_scan);
 }

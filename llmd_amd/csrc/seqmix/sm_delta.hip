@@ -69,6 +69,33 @@ __global__ __launch_bounds__(NT) void delta_prep_kernel(const T* __restrict__ xc
   }
 }
 
+// HGRN2: queries, gates and write strengths of every token (fp32), from the projection [q | f | ...].
+// qn = silu(q), dec = f = lower + (1 - lower) sigmoid(f_raw + bias), kn = 1 - f; all [T, H, KD].
+// Rows beyond dk: q = k = 0, f = 1.
+template <typename T>
+__global__ __launch_bounds__(NT) void hgrn2_prep_kernel(const T* __restrict__ p, int64_t p_stride, int H, int dk,
+                                                       int KD, const float* __restrict__ f_bias,
+                                                       const float* __restrict__ lower, float* __restrict__ qn,
+                                                       float* __restrict__ kn, float* __restrict__ dec) {
+  const int64_t t = blockIdx.x;
+  const T* pr = p + t * p_stride;
+  for (int idx = blockIdx.y * NT + threadIdx.x; idx < H * KD; idx += gridDim.y * NT) {
+    const int h = idx / KD, i = idx - h * KD;
+    float q = 0.f, k = 0.f, f = 1.f;
+    if (i < dk) {
+      const int c = h * dk + i;
+      q = Fn<T>::silu(ld(pr + c));
+      const float lo = lower[c];
+      const float sg = Fn<T>::sigmoid(ld(pr + H * dk + c) + f_bias[c]);
+      f = lo + (1.f - lo) * sg;
+      k = (1.f - lo) * (1.f - sg);  // 1 - f without the cancellation near f = 1
+    }
+    qn[t * H * KD + idx] = q;
+    kn[t * H * KD + idx] = k;
+    dec[t * H * KD + idx] = f;
+  }
+}
+
 // Sum over the RG (4 or 8) neighbouring lanes of a column (lanes RG c .. RG c + RG - 1): DPP
 // exchanges, no LDS. After the two quad exchanges all four lanes of a quad hold the quad's sum; the
 // mirror inside a half row (lane i <-> 7 - i) then brings the other quad's.
@@ -87,7 +114,7 @@ __device__ __forceinline__ float group_sum(float v) {
 // tokens from one buffer, the next block's loads are in flight into registers, and are written to the
 // other buffer afterwards - the recurrence never waits for global memory. Per token a lane reads its
 // KR rows of k, q (and g) as 16-byte LDS broadcasts.
-template <typename T, int KR, int RG, bool CH, int TB>
+template <typename T, int KR, int RG, bool CH, int TB, bool DELTA = true>
 __global__ __launch_bounds__(64) void gated_delta_scan_kernel(
     const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ dec,
     const float* __restrict__ beta, const T* __restrict__ xc, int64_t x_stride, int voff, int G, int dk, int H, int dv,
@@ -125,13 +152,15 @@ __global__ __launch_bounds__(64) void gated_delta_scan_kernel(
       } else {
         S[i] *= gj; S[i + 1] *= gj; S[i + 2] *= gj; S[i + 3] *= gj;
       }
-      p[0] += k[i] * S[i];
-      p[1] += k[i + 1] * S[i + 1];
-      p[2] += k[i + 2] * S[i + 2];
-      p[3] += k[i + 3] * S[i + 3];
+      if (DELTA) {
+        p[0] += k[i] * S[i];
+        p[1] += k[i + 1] * S[i + 1];
+        p[2] += k[i + 2] * S[i + 2];
+        p[3] += k[i + 3] * S[i + 3];
+      }
     }
-    const float pred = group_sum<RG>((p[0] + p[1]) + (p[2] + p[3]));
-    const float u = bj * (vj - pred);
+    const float pred = DELTA ? group_sum<RG>((p[0] + p[1]) + (p[2] + p[3])) : 0.f;
+    const float u = DELTA ? bj * (vj - pred) : vj;
     float o[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < KR; i += 4) {
@@ -151,7 +180,7 @@ __global__ __launch_bounds__(64) void gated_delta_scan_kernel(
       const float4* qp = reinterpret_cast<const float4*>(qn + (t * G + qh) * KD + row0);
       const float4* gp = reinterpret_cast<const float4*>(CH ? dec + (t * H + h) * KD + row0 : kn);
       const float vj = colok ? ld(xc + t * x_stride + voff + h * dv + col) : 0.f;
-      const float ov = token(kp, qp, gp, CH ? 1.f : dec[t * H + h], beta[t * H + h], vj);
+      const float ov = token(kp, qp, gp, CH ? 1.f : dec[t * H + h], DELTA ? beta[t * H + h] : 1.f, vj);
       if (r == 0 && colok) o_raw[t * H * dv + h * dv + col] = ov;
     }
   } else {
@@ -179,7 +208,7 @@ __global__ __launch_bounds__(64) void gated_delta_scan_kernel(
         if (!CH) gb[j] = 1.f;
         if (t >= hi) continue;
         vb[j] = colok ? ld(xc + t * x_stride + voff + h * dv + col) : 0.f;
-        bb[j] = beta[t * H + h];
+        bb[j] = DELTA ? beta[t * H + h] : 1.f;
         if (!CH) gb[j] = dec[t * H + h];
       }
     };
@@ -236,8 +265,11 @@ __global__ __launch_bounds__(NT) void delta_out_kernel(const float* __restrict__
     for (int e = lane; e < dv; e += 64) ss += orow[e] * orow[e];
     const float inv = Fn<T>::rsqrt(wave_sum(ss) / (float)dv + eps);
     for (int e = lane; e < dv; e += 64) {
-      const float gr = ld(gate_raw + t * gate_stride + h * dv + e);
-      const float gt = gate_sigmoid ? Fn<T>::sigmoid(gr) : Fn<T>::silu(gr);
+      float gt = 1.f;  // no gate: the norm alone
+      if (gate_raw != nullptr) {
+        const float gr = ld(gate_raw + t * gate_stride + h * dv + e);
+        gt = gate_sigmoid ? Fn<T>::sigmoid(gr) : Fn<T>::silu(gr);
+      }
       st(out + (t * H + h) * dv + e, orow[e] * inv * ld(norm_w + e) * gt);
     }
   }
@@ -292,6 +324,45 @@ int sm_gated_delta_scan(const void* xc, int64_t x_stride, int G, int dk, int H, 
   else { SM_ALL(bf16_t); }
 #undef SM_ALL
 #undef SM_KR
+#undef SM_RG
+#undef SM_GO
+  return 0;
+}
+
+// HGRN2 over the projection p = [q | f | v] (H dk, H dk, H dv columns). Workspaces (fp32): qn, kn, dec
+// [T, H, KD]; o_raw [T, H, dv]. Returns 0, or 1 when the key size does not fit (dk > 256).
+int sm_hgrn2_scan(const void* p, int64_t p_stride, int H, int dk, int dv, const float* f_bias, const float* lower,
+                  const void* norm_w, float eps, float* state, const int* seq_start, const int* seq_slot,
+                  const int* seq_init, void* out, float* qn, float* kn, float* dec, float* o_raw, int T, int nseq,
+                  int f32, hipStream_t stream) {
+  if (nseq == 0 || T == 0) return 0;
+  const int KD = sm_gated_delta_rows(dk);
+  if (KD == 0) return 1;
+  const int voff = 2 * H * dk;
+  const bool wide = (int64_t)nseq * H * ((dv + 15) / 16) >= 1024;
+  const int cpw = wide ? 16 : 8;
+  const dim3 grid(H * ((dv + cpw - 1) / cpw), nseq);
+  const dim3 pgrid(T, std::max(1, std::min((H * KD + NT - 1) / NT, 4096 / T)));
+  const dim3 ogrid(T, std::max(1, std::min((H + 3) / 4, 4096 / T)));
+#define SM_GO(TYPE, KR, RG)                                                                                          \
+  hipLaunchKernelGGL((gated_delta_scan_kernel<TYPE, KR, RG, true, (KR * RG <= 128 ? 16 : 8), false>), grid, dim3(64), \
+                     0, stream, qn, kn, dec, nullptr, (const TYPE*)p, p_stride, voff, H, dk, H, dv, state, seq_start, \
+                     seq_slot, seq_init, o_raw)
+#define SM_RG(TYPE, KD_)              \
+  if (wide) SM_GO(TYPE, KD_ / 4, 4);  \
+  else SM_GO(TYPE, KD_ / 8, 8)
+#define SM_ALL(TYPE)                                                                                                 \
+  hipLaunchKernelGGL((hgrn2_prep_kernel<TYPE>), pgrid, dim3(NT), 0, stream, (const TYPE*)p, p_stride, H, dk, KD,      \
+                     f_bias, lower, qn, kn, dec);                                                                    \
+  if (KD == 32) { SM_RG(TYPE, 32); }                                                                                 \
+  else if (KD == 64) { SM_RG(TYPE, 64); }                                                                            \
+  else if (KD == 128) { SM_RG(TYPE, 128); }                                                                          \
+  else { SM_RG(TYPE, 256); }                                                                                         \
+  hipLaunchKernelGGL((delta_out_kernel<TYPE>), ogrid, dim3(NT), 0, stream, o_raw, (const TYPE*)nullptr, (int64_t)0, 0, \
+                     (const TYPE*)norm_w, eps, H, dv, (TYPE*)out)
+  if (f32) { SM_ALL(float); }
+  else { SM_ALL(bf16_t); }
+#undef SM_ALL
 #undef SM_RG
 #undef SM_GO
   return 0;

@@ -1,7 +1,8 @@
 // Row kernels of per-layer stacks: embedding with scale, zero-centred RMS norms on the fp32
 // residual, post-norm + layer scale + residual add (+ the next pre-norm in the same pass),
 // the depth average (+ the norm that follows it), xIELU and the logit soft cap; the embedding with
-// a hashed bigram table and the plain post-norm residual add of stacks that norm only outputs.
+// a hashed bigram table and the plain post-norm residual add of stacks that norm only outputs; the
+// embedding with the first plain norm, the plain norm of a projection's rows and the squared ReLU.
 // One workgroup of 256 threads per token row; the fp32 residual is read and written once.
 #include "seqmix_common.h"
 
@@ -191,9 +192,109 @@ __global__ __launch_bounds__(NT) void post_norm_add_kernel(const T* __restrict__
   for (int c = threadIdx.x; c < d; c += NT) st(out + row * d + c, xr[c] * inv2 * ld(wn + c));
 }
 
+// x = table[id] (fp32 residual);  out = x / rms(x) * w
+template <typename T>
+__global__ __launch_bounds__(NT) void embed_norm_kernel(const int64_t* __restrict__ ids, const T* __restrict__ table,
+                                                       int64_t V, const T* __restrict__ w, float eps,
+                                                       float* __restrict__ x, T* __restrict__ out, int d) {
+  __shared__ float red[NT / 64];
+  const int64_t row = blockIdx.x;
+  const int64_t id = min(max(ids[row], (int64_t)0), V - 1);  // a bad id must not read outside the table
+  const T* src = table + id * (int64_t)d;
+  float* xr = x + row * d;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < d; c += NT) {
+    const float v = ld(src + c);
+    xr[c] = v;
+    ss += v * v;
+  }
+  ss = block_sum<NT>(ss, red);
+  const float inv = 1.f / sqrtf(ss / (float)d + eps);
+  for (int c = threadIdx.x; c < d; c += NT) st(out + row * d + c, ld(src + c) * inv * ld(w + c));
+}
+
+// out = y / rms(y) * w over rows of n elements (y may be a column view: y_stride); a wave per row
+template <typename T>
+__global__ __launch_bounds__(NT) void rms_norm_rows_kernel(const T* __restrict__ y, int64_t y_stride,
+                                                          const T* __restrict__ w, float eps, T* __restrict__ out,
+                                                          int n, int rows) {
+  const int64_t row = (int64_t)blockIdx.x * (NT / 64) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const T* yr = y + row * y_stride;
+  float ss = 0.f;
+  for (int c = lane; c < n; c += 64) {
+    const float v = ld(yr + c);
+    ss += v * v;
+  }
+  const float inv = 1.f / sqrtf(wave_sum(ss) / (float)n + eps);
+  for (int c = lane; c < n; c += 64) st(out + row * n + c, ld(yr + c) * inv * ld(w + c));
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void relu2_kernel(const T* __restrict__ z, T* __restrict__ out, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * NT + threadIdx.x;
+  if (i >= n) return;
+  const float v = fmaxf(ld(z + i), 0.f);
+  st(out + i, v * v);
+}
+
+// bf16, eight elements per thread (n a multiple of 8, 16-byte aligned)
+__global__ __launch_bounds__(NT) void relu2_vec_kernel(const uint4* __restrict__ z, uint4* __restrict__ out, int64_t n8) {
+  const int64_t i = (int64_t)blockIdx.x * NT + threadIdx.x;
+  if (i >= n8) return;
+  const uint4 t = z[i];
+  uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const float a = fmaxf(__uint_as_float(w[k] << 16), 0.f), b = fmaxf(__uint_as_float(w[k] & 0xffff0000u), 0.f);
+    const __bf16 ha = (__bf16)(a * a), hb = (__bf16)(b * b);
+    w[k] = (uint32_t)__builtin_bit_cast(uint16_t, ha) | ((uint32_t)__builtin_bit_cast(uint16_t, hb) << 16);
+  }
+  out[i] = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
 }  // namespace
 
 extern "C" {
+
+void sm_embed_norm(const int64_t* ids, const void* table, int64_t V, const void* w, float eps, float* x, void* out,
+                   int T, int d, int f32, hipStream_t stream) {
+  if (T == 0) return;
+  if (f32)
+    hipLaunchKernelGGL((embed_norm_kernel<float>), dim3(T), dim3(NT), 0, stream, ids, (const float*)table, V,
+                       (const float*)w, eps, x, (float*)out, d);
+  else
+    hipLaunchKernelGGL((embed_norm_kernel<bf16_t>), dim3(T), dim3(NT), 0, stream, ids, (const bf16_t*)table, V,
+                       (const bf16_t*)w, eps, x, (bf16_t*)out, d);
+}
+
+void sm_rms_norm_rows(const void* y, int64_t y_stride, const void* w, float eps, void* out, int rows, int n, int f32,
+                      hipStream_t stream) {
+  if (rows == 0) return;
+  const dim3 grid((rows + NT / 64 - 1) / (NT / 64));
+  if (f32)
+    hipLaunchKernelGGL((rms_norm_rows_kernel<float>), grid, dim3(NT), 0, stream, (const float*)y, y_stride,
+                       (const float*)w, eps, (float*)out, n, rows);
+  else
+    hipLaunchKernelGGL((rms_norm_rows_kernel<bf16_t>), grid, dim3(NT), 0, stream, (const bf16_t*)y, y_stride,
+                       (const bf16_t*)w, eps, (bf16_t*)out, n, rows);
+}
+
+void sm_relu2(const void* z, void* out, int64_t n, int f32, hipStream_t stream) {
+  if (n == 0) return;
+  if (f32) {
+    hipLaunchKernelGGL((relu2_kernel<float>), dim3((unsigned)((n + NT - 1) / NT)), dim3(NT), 0, stream,
+                       (const float*)z, (float*)out, n);
+  } else if ((n & 7) == 0 && (((uintptr_t)z | (uintptr_t)out) & 15) == 0) {
+    const int64_t n8 = n >> 3;
+    hipLaunchKernelGGL(relu2_vec_kernel, dim3((unsigned)((n8 + NT - 1) / NT)), dim3(NT), 0, stream, (const uint4*)z,
+                       (uint4*)out, n8);
+  } else {
+    hipLaunchKernelGGL((relu2_kernel<bf16_t>), dim3((unsigned)((n + NT - 1) / NT)), dim3(NT), 0, stream,
+                       (const bf16_t*)z, (bf16_t*)out, n);
+  }
+}
 
 void sm_bigram_embed(const int64_t* ids, const void* table, float scale, int64_t V, const void* bigram,
                      int64_t buckets, int64_t mul_prev, int64_t mul_cur, int* prev_state, const int* row_seq,

@@ -25,6 +25,10 @@
 // score per head that enters the softmax's denominator and has no value (the running maximum and
 // sum start from it instead of from nothing). Key tiles start at multiples of the tile size from
 // position 0, so a row's tiles do not depend on what else the step holds.
+// window / keep: query i sees key j <= i only if i - j < window or j < keep (the sequence's first
+// tokens stay visible); the tiles between the kept tokens and the first window of a work item are
+// skipped. qkv_rope_cache options: norm_first - the unit norm and its weights come before the
+// rotation; v_from_k - the values are the biased key projections themselves (no value columns).
 #include "seqmix_common.h"
 #include <algorithm>
 
@@ -40,7 +44,8 @@ __global__ __launch_bounds__(NT) void qkv_rope_cache_kernel(
     const T* __restrict__ qkv, int64_t stride, const float* __restrict__ bias, const int64_t* __restrict__ positions,
     const float* __restrict__ cos_sin, int Hq, int Hkv, int dim, int vdim, int rot_dims, int interleaved, int unit,
     float eps, float* __restrict__ v_first, int v_mode, float lam, const int64_t* __restrict__ slots,
-    T* __restrict__ cache, int bs, T* __restrict__ q_out, const float* __restrict__ qk_w) {
+    T* __restrict__ cache, int bs, T* __restrict__ q_out, const float* __restrict__ qk_w, int norm_first,
+    int v_from_k) {
   const int64_t t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int half = rot_dims >> 1;
@@ -54,14 +59,17 @@ __global__ __launch_bounds__(NT) void qkv_rope_cache_kernel(
   for (int hd = blockIdx.y * (NT / 64) + wave; hd < Hq + Hkv; hd += gridDim.y * (NT / 64)) {
     const bool is_q = hd < Hq;
     const int col0 = is_q ? hd * dim : Hq * dim + (hd - Hq) * dim;
+    const float* nw = qk_w ? qk_w + (is_q ? 0 : dim) : nullptr;  // the norm's weight, shared by the heads
+    const float* nw1 = norm_first ? nw : nullptr;               // applied before the rotation
     float r[MAXE];
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < MAXE; ++i) {
       const int e = lane + 64 * i;
-      float v = 0.f;
+      float v = 0.f, raw = 0.f;
       if (e < dim) {
-        const float x = ld(row + col0 + e) + (bias ? bias[col0 + e] : 0.f);
+        raw = ld(row + col0 + e) + (bias ? bias[col0 + e] : 0.f);
+        const float x = nw1 ? raw * nw1[e] : raw;
         v = x;
         if (e < rot_dims) {
           int p, f;
@@ -75,13 +83,13 @@ __global__ __launch_bounds__(NT) void qkv_rope_cache_kernel(
             p = first ? e + half : e - half;
             f = first ? e : e - half;
           }
-          const float xp = ld(row + col0 + p) + (bias ? bias[col0 + p] : 0.f);
+          const float xp = (ld(row + col0 + p) + (bias ? bias[col0 + p] : 0.f)) * (nw1 ? nw1[p] : 1.f);
           const float c = cs[f], s = cs[half + f];
           v = first ? x * c - xp * s : x * c + xp * s;
         }
       }
       r[i] = v;
-      ss += v * v;
+      ss += norm_first ? raw * raw : v * v;
     }
     float inv = 1.f;
     if (unit) inv = 1.f / sqrtf(wave_sum(ss) / (float)dim + eps);
@@ -89,14 +97,13 @@ __global__ __launch_bounds__(NT) void qkv_rope_cache_kernel(
     if (is_q) dst = q_out + (t * Hq + hd) * dim;
     else if (slot >= 0) dst = cache + (blk * Hkv + (hd - Hq)) * bs * Dr + off * dim;
     if (dst == nullptr) continue;
-    const float* nw = qk_w ? qk_w + (is_q ? 0 : dim) : nullptr;  // the norm's weight, shared by the heads
 #pragma unroll
     for (int i = 0; i < MAXE; ++i) {
       const int e = lane + 64 * i;
-      if (e < dim) st(dst + e, r[i] * inv * (nw ? nw[e] : 1.f));
+      if (e < dim) st(dst + e, r[i] * inv * ((nw && !norm_first) ? nw[e] : 1.f));
     }
   }
-  const int nv = Hkv * vdim, vcol0 = (Hq + Hkv) * dim;
+  const int nv = Hkv * vdim, vcol0 = v_from_k ? Hq * dim : (Hq + Hkv) * dim;
   for (int e = blockIdx.y * NT + threadIdx.x; e < nv; e += gridDim.y * NT) {
     float v = ld(row + vcol0 + e) + (bias ? bias[vcol0 + e] : 0.f);
     if (v_mode == 1) v_first[t * nv + e] = v;
@@ -141,7 +148,7 @@ __global__ __launch_bounds__(NT) void qkv_rope_cache_vec_kernel(
     const int64_t* __restrict__ positions, const float* __restrict__ cos_sin, int Hq, int Hkv, int dim, int vdim,
     int rot_dims, int interleaved, int unit, float eps, float* __restrict__ v_first, int v_mode, float lam,
     const int64_t* __restrict__ slots, bf16_t* __restrict__ cache, int bs, bf16_t* __restrict__ q_out,
-    const float* __restrict__ qk_w) {
+    const float* __restrict__ qk_w, int norm_first, int v_from_k) {
   const int64_t t = blockIdx.x;
   const int half = rot_dims >> 1;
   const float* cs = rot_dims ? cos_sin + positions[t] * rot_dims : nullptr;  // [cos(half) | sin(half)]
@@ -156,9 +163,19 @@ __global__ __launch_bounds__(NT) void qkv_rope_cache_vec_kernel(
     const bool on = hd < Hq + Hkv;
     const int col = hd * dim + c * 8;  // q heads, then k heads, back to back in the projection
     float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    float ss = 0.f;
+    const float* nw = qk_w ? qk_w + (hd < Hq ? 0 : dim) : nullptr;
+    const float* nw1 = norm_first ? nw : nullptr;  // weights applied before the rotation
     if (on) {
       ld8(row + col, x);
       if (bias) add8(bias + col, x);
+      if (norm_first) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          ss += x[i] * x[i];
+          if (nw1) x[i] *= nw1[c * 8 + i];
+        }
+      }
       if (c * 8 < rot_dims) {
         if (interleaved) {
           const float4 co = *reinterpret_cast<const float4*>(cs + c * 4);
@@ -177,6 +194,10 @@ __global__ __launch_bounds__(NT) void qkv_rope_cache_vec_kernel(
           float xp[8], cc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, sn[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
           ld8(row + pc, xp);
           if (bias) add8(bias + pc, xp);
+          if (nw1) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) xp[i] *= nw1[c * 8 + (first ? half : -half) + i];
+          }
           add8(cs + f, cc);
           add8(cs + half + f, sn);
 #pragma unroll
@@ -186,22 +207,22 @@ __global__ __launch_bounds__(NT) void qkv_rope_cache_vec_kernel(
     }
     float inv = 1.f;
     if (unit) {
-      float ss = 0.f;
+      if (!norm_first) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) ss += x[i] * x[i];
+        for (int i = 0; i < 8; ++i) ss += x[i] * x[i];
+      }
       for (int o = lph >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);  // the head's lanes are an aligned group
       inv = 1.f / sqrtf(ss / (float)dim + eps);
     }
     if (!on) continue;
-    if (qk_w) {
-      const float* nw = qk_w + (hd < Hq ? 0 : dim) + c * 8;
+    if (nw && !norm_first) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) x[i] *= nw[i];
+      for (int i = 0; i < 8; ++i) x[i] *= nw[c * 8 + i];
     }
     if (hd < Hq) st8(q_out + (t * Hq + hd) * dim + c * 8, x, inv);
     else if (slot >= 0) st8(cache + (blk * Hkv + (hd - Hq)) * bs * Dr + off * dim + c * 8, x, inv);
   }
-  const int nv = Hkv * vdim, vcol0 = (Hq + Hkv) * dim;
+  const int nv = Hkv * vdim, vcol0 = v_from_k ? Hq * dim : (Hq + Hkv) * dim;
   for (int e = blockIdx.y * NT + threadIdx.x; e < nv; e += gridDim.y * NT) {
     float v = ld(row + vcol0 + e) + (bias ? bias[vcol0 + e] : 0.f);
     if (v_mode == 1) v_first[t * nv + e] = v;
@@ -219,7 +240,7 @@ __global__ __launch_bounds__(NT) void grouped_attention_kernel(
     const T* __restrict__ q, const T* __restrict__ cache, const int* __restrict__ tables, int W, int bs,
     const int* __restrict__ row_seq, const int* __restrict__ row_len, float scale, int Hq, int Hkv, int dim, int vdim,
     int KT, int T_rows, const T* __restrict__ gate, int64_t gate_stride, T* __restrict__ out,
-    const float* __restrict__ slopes, int chunk, const float* __restrict__ sinks) {
+    const float* __restrict__ slopes, int chunk, const float* __restrict__ sinks, int window, int keep) {
   extern __shared__ float lds[];
   const int Dr = dim + vdim;
   const int KS = Dr + 1;                 // tile row stride (odd: lanes hit distinct banks)
@@ -240,8 +261,9 @@ __global__ __launch_bounds__(NT) void grouped_attention_kernel(
     sQ[e] = (t < T_rows && hh < G) ? ld(q + ((int64_t)t * Hq + g * G + hh) * dim + d) * scale : 0.f;
   }
 
-  int seq_r[QT], len_r[QT], lo_r[QT];
+  int seq_r[QT], len_r[QT], lo_r[QT], wlo_r[QT];
   bool done[QT];
+  if (window <= 0) keep = 0;
 #pragma unroll
   for (int r = 0; r < QT; ++r) {
     const int t = t0 + r;
@@ -249,6 +271,7 @@ __global__ __launch_bounds__(NT) void grouped_attention_kernel(
     seq_r[r] = done[r] ? -1 : row_seq[t];
     len_r[r] = done[r] ? 0 : row_len[t];
     lo_r[r] = (chunk > 0 && len_r[r] > 0) ? ((len_r[r] - 1) / chunk) * chunk : 0;  // first key of the row's chunk
+    wlo_r[r] = window > 0 ? max(0, len_r[r] - window) : 0;                          // first key of the row's window
   }
   const float slope = (slopes != nullptr && head_ok) ? slopes[h] : 0.f;
   const bool has_sink = sinks != nullptr && head_ok;
@@ -261,13 +284,14 @@ __global__ __launch_bounds__(NT) void grouped_attention_kernel(
       if (seq < 0 && !done[r]) seq = seq_r[r];
     if (seq < 0) break;
     bool act[QT];
-    int maxlen = 0, minlo = 0x7fffffff;
+    int maxlen = 0, minlo = 0x7fffffff, minwlo = 0x7fffffff;
 #pragma unroll
     for (int r = 0; r < QT; ++r) {
       act[r] = !done[r] && seq_r[r] == seq;
       if (act[r]) {
         maxlen = max(maxlen, len_r[r]);
         minlo = min(minlo, lo_r[r]);
+        minwlo = min(minwlo, wlo_r[r]);
       }
     }
     float m[QT], l[QT], acc[QT][VC];
@@ -279,7 +303,11 @@ __global__ __launch_bounds__(NT) void grouped_attention_kernel(
       for (int c = 0; c < VC; ++c) acc[r][c] = 0.f;
     }
     const int* bt = tables + (int64_t)seq * W;
+    bool first_tile = true;
     for (int k0 = (minlo / KT) * KT; k0 < maxlen; k0 += KT) {
+      // a tile past the kept first tokens and before every row's window holds nothing visible
+      if (!first_tile && k0 >= keep && k0 + KT <= minwlo) continue;
+      first_tile = false;  // the first pass always runs: its barrier orders the query tile's writes
       __syncthreads();  // previous tile fully used (and sQ written, first time)
       for (int e = threadIdx.x; e < KT * dim; e += NT) {  // keys: row-major in the page
         const int j = e / dim, d = e - j * dim;
@@ -300,8 +328,9 @@ __global__ __launch_bounds__(NT) void grouped_attention_kernel(
       if (!head_ok) continue;
 #pragma unroll
       for (int r = 0; r < QT; ++r) {
-        if (!act[r] || k0 >= len_r[r] || k0 + KT <= lo_r[r]) continue;
-        const bool valid = lane < KT && k0 + lane < len_r[r] && k0 + lane >= lo_r[r];
+        if (!act[r] || k0 >= len_r[r] || k0 + KT <= lo_r[r] || (k0 >= keep && k0 + KT <= wlo_r[r])) continue;
+        const bool valid = lane < KT && k0 + lane < len_r[r] && k0 + lane >= lo_r[r] &&
+                           (k0 + lane >= wlo_r[r] || k0 + lane < keep);
         float s = -INFINITY;
         if (valid) {
           const float* qv = sQ + (r * 4 + wave) * dim;
@@ -365,7 +394,7 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
     const int* __restrict__ items, const int* __restrict__ row_len, float scale, int Hq, int Hkv, int dim, int vdim,
     const bf16_t* __restrict__ gate, int64_t gate_stride, bf16_t* __restrict__ out, int split_keys,
     float* __restrict__ part_o, float* __restrict__ part_ml, const float* __restrict__ slopes, int chunk,
-    const float* __restrict__ sinks) {
+    const float* __restrict__ sinks, int window, int keep) {
   constexpr int DkP = 32 * NKS, VP = 16 * NCB;
   constexpr int KS = DkP + 8, VS = MKT + 8;  // LDS row strides (bf16), 16-byte multiples
   // Two tile buffers for the small forms: the next tile is written while the current one is read and
@@ -380,8 +409,9 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r16 = lane & 15, kq = lane >> 4;
   // this lane's query rows (as the B operand's column): item row 16 (4 rb + wave) + r16
-  int mytok[RB], myhead[RB], mylen[RB], mylo[RB];
+  int mytok[RB], myhead[RB], mylen[RB], mylo[RB], mywlo[RB];
   float myslope[RB];  // in base 2, like the scores
+  if (window <= 0) keep = 0;
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const int myrow = (rb * 4 + wave) * 16 + r16;
@@ -390,11 +420,23 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
     myhead[rb] = g * G + (ok ? myrow % G : 0);
     mylen[rb] = ok ? row_len[mytok[rb]] : 0;
     mylo[rb] = (chunk > 0 && mylen[rb] > 0) ? ((mylen[rb] - 1) / chunk) * chunk : 0;  // first key of the row's chunk
+    mywlo[rb] = window > 0 ? max(0, mylen[rb] - window) : 0;                             // first key of the row's window
     myslope[rb] = slopes ? slopes[myhead[rb]] * 1.44269504088896341f : 0.f;
   }
   const int maxlen = row_len[tok0 + ntok - 1];  // the run's last token sees the most keys
   // the run's first token starts the earliest chunk; tiles start at multiples of 32 from position 0
   const int kbase = chunk > 0 ? ((((row_len[tok0] - 1) / chunk) * chunk) / MKT) * MKT : 0;
+  // A window leaves a gap between the tiles of the kept first tokens [0, keepT) and the tile that the
+  // run's first window starts in. The tile loop runs over positions v with the gap taken out:
+  // key = v below keepT, v + gap from there on; the decode split cuts [0, vlen) too.
+  int keepT = 0, gap = 0;
+  if (window > 0) {
+    keepT = ((keep + MKT - 1) / MKT) * MKT;
+    const int wbase = (max(0, row_len[tok0] - window) / MKT) * MKT;
+    gap = max(0, wbase - keepT);
+  }
+  const int vlen = maxlen - gap;
+  auto key_of = [&](int v) { return v + (v >= keepT ? gap : 0); };
 
   // padding columns of the key tile and padding rows of the value tile stay zero for the whole kernel
   for (int e = threadIdx.x; e < NBUF * MKT * KS; e += NT) sK[e] = 0;
@@ -431,8 +473,9 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
 
   // decode steps split a row's keys over blockIdx.z: this workgroup takes [kbeg, kend)
   const int nsplit = gridDim.z;
+  // (ranges are whole tiles, so a tile's keys need only stay below maxlen)
   const int kbeg = nsplit > 1 ? kbase + blockIdx.z * split_keys : kbase;
-  const int kend = nsplit > 1 ? min(maxlen, kbeg + split_keys) : maxlen;
+  const int kend = nsplit > 1 ? min(vlen, kbeg + split_keys) : vlen;
   constexpr int CK = DkP / 8;                      // 16-byte chunks per key row (padded)
   constexpr int NCK = (MKT * CK + NT - 1) / NT;    // key chunks per thread
   constexpr int CV = MKT / 8;                      // chunks per value column (8 keys each)
@@ -443,8 +486,13 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
   // kend are zeroed (a page's unwritten rest may hold anything, and 0 x NaN would spoil a column).
   u32x4_t pk[NCK], pv[NCV];
   // one-page tiles: the tile's page and its first row in the page advance without a division
-  int tile_page = one_page ? kbeg / bs : 0, tile_off = one_page ? kbeg % bs : 0;
+  int tile_page = 0, tile_off = 0, tile_next = -1;
   auto fetch = [&](int k0) {
+    if (one_page && k0 != tile_next) {  // the first tile, and the one after the gap
+      tile_page = k0 / bs;
+      tile_off = k0 % bs;
+    }
+    tile_next = k0 + MKT;
     const int64_t page0 = one_page ? ((int64_t)bt[tile_page] * Hkv + g) * bs * Dr : 0;
     const int off0 = tile_off;
     if (one_page) {
@@ -460,7 +508,7 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
       const int j = e / CK, c = e - j * CK;
       const int key = k0 + j;
       u32x4_t v = {0, 0, 0, 0};
-      if (e < MKT * CK && c * 8 < dim && key < kend) {
+      if (e < MKT * CK && c * 8 < dim && key < maxlen) {
         const int64_t page = one_page ? page0 : ((int64_t)bt[key / bs] * Hkv + g) * bs * Dr;
         const int off = one_page ? off0 + j : key % bs;
         const bf16_t* src = cache + page + (int64_t)off * dim + c * 8;
@@ -480,11 +528,11 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
       const int d = e / CV, j8 = e - d * CV;
       const int key = k0 + j8 * 8;
       u32x4_t v = {0, 0, 0, 0};
-      if (d < vdim && key < kend) {
+      if (d < vdim && key < maxlen) {
         const int64_t page = one_page ? page0 : ((int64_t)bt[key / bs] * Hkv + g) * bs * Dr;
         const int off = one_page ? off0 + j8 * 8 : key % bs;
         v = *reinterpret_cast<const u32x4_t*>(cache + page + (int64_t)bs * dim + (int64_t)d * bs + off);
-        const int nv = kend - key;  // keys of this chunk that exist
+        const int nv = maxlen - key;  // keys of this chunk that exist
         if (nv < 8) {
 #pragma unroll
           for (int w = 0; w < 4; ++w) v[w] = 2 * w + 1 < nv ? v[w] : (2 * w < nv ? v[w] & 0xffffu : 0u);
@@ -515,21 +563,22 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
       }
     }
   };
-  if (kbeg < kend) fetch(kbeg);
+  if (kbeg < kend) fetch(key_of(kbeg));
   if (NBUF == 2) {
     __syncthreads();  // the zero fill is done
     stage(0);
-    if (kbeg + MKT < kend) fetch(kbeg + MKT);
+    if (kbeg + MKT < kend) fetch(key_of(kbeg + MKT));
     __syncthreads();
   }
   int it = 0;
-  for (int k0 = kbeg; k0 < kend; k0 += MKT, ++it) {
+  for (int v0 = kbeg; v0 < kend; v0 += MKT, ++it) {
+    const int k0 = key_of(v0);
     const int cur = NBUF == 2 ? (it & 1) : 0;
     if (NBUF == 1) {
       __syncthreads();  // the previous tile is no longer read (first time: the zero fill is done)
       stage(0);
       __syncthreads();
-      if (k0 + MKT < kend) fetch(k0 + MKT);  // in flight during this tile's products
+      if (v0 + MKT < kend) fetch(key_of(v0 + MKT));  // in flight during this tile's products
     }
     const bf16_t* const tK = sK + cur * MKT * KS;
     const bf16_t* const tV = sVt + cur * VP * VS;
@@ -551,7 +600,7 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int key = k0 + kb * 16 + kq * 4 + r;
-          sc[rb][kb][r] = (key < min(mylen[rb], kend) && key >= mylo[rb])
+          sc[rb][kb][r] = (key < mylen[rb] && key >= mylo[rb] && (key >= mywlo[rb] || key < keep))
                               ? a[rb][r] * scale2 - myslope[rb] * (float)(mylen[rb] - 1 - key)
                               : -INFINITY;
         }
@@ -623,9 +672,9 @@ __global__ __launch_bounds__(NT) void grouped_attention_mfma_kernel(
     if (NBUF == 2) {
       // every wave has finished the previous tile (barrier below, one iteration ago), so the other
       // buffer is free: write the next tile there and ask for the one after it
-      if (k0 + MKT < kend) {
+      if (v0 + MKT < kend) {
         stage(cur ^ 1);
-        if (k0 + 2 * MKT < kend) fetch(k0 + 2 * MKT);
+        if (v0 + 2 * MKT < kend) fetch(key_of(v0 + 2 * MKT));
       }
       __syncthreads();
     }
@@ -705,7 +754,7 @@ template <typename T, int VC>
 int launch_attn(const void* q, const void* cache, const int* tables, int W, int bs, const int* row_seq,
                 const int* row_len, float scale, int Hq, int Hkv, int dim, int vdim, int T_rows, int QT,
                 const void* gate, int64_t gate_stride, void* out, const float* slopes, int chunk, const float* sinks,
-                hipStream_t stream) {
+                int window, int keep, hipStream_t stream) {
   const int Dr = dim + vdim;
   int KT = 64;
   while (KT > 16 && ((size_t)KT * (Dr + 1) + (size_t)QT * 4 * dim) * 4 > 128 * 1024) KT >>= 1;
@@ -716,7 +765,8 @@ int launch_attn(const void* q, const void* cache, const int* tables, int W, int 
   auto go = [&](auto kern) {
     if (lds > 64 * 1024) (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(kern, grid, dim3(NT), lds, stream, (const T*)q, (const T*)cache, tables, W, bs, row_seq, row_len,
-                       scale, Hq, Hkv, dim, vdim, KT, T_rows, (const T*)gate, gate_stride, (T*)out, slopes, chunk, sinks);
+                       scale, Hq, Hkv, dim, vdim, KT, T_rows, (const T*)gate, gate_stride, (T*)out, slopes, chunk, sinks,
+                       window, keep);
   };
   if (QT == 4) go(grouped_attention_kernel<T, VC, 4>);
   else go(grouped_attention_kernel<T, VC, 1>);
@@ -730,7 +780,8 @@ extern "C" {
 void sm_qkv_rope_cache(const void* qkv, int64_t stride, const float* bias, const int64_t* positions,
                        const float* cos_sin, int Hq, int Hkv, int dim, int vdim, int rot_dims, int interleaved,
                        int unit, float eps, float* v_first, int v_mode, float lam, const int64_t* slots, void* cache,
-                       int bs, void* q_out, const float* qk_w, int T, int f32, hipStream_t stream) {
+                       int bs, void* q_out, const float* qk_w, int norm_first, int v_from_k, int T, int f32,
+                       hipStream_t stream) {
   if (T == 0) return;
   // workgroups per token: all heads in parallel for small steps, fewer as the step grows
   const int per_tok = (Hq + Hkv + NT / 64 - 1) / (NT / 64);
@@ -739,7 +790,7 @@ void sm_qkv_rope_cache(const void* qkv, int64_t stride, const float* bias, const
   if (f32)
     hipLaunchKernelGGL((qkv_rope_cache_kernel<float>), grid, dim3(NT), 0, stream, (const float*)qkv, stride, bias,
                        positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit, eps, v_first, v_mode, lam,
-                       slots, (float*)cache, bs, (float*)q_out, qk_w);
+                       slots, (float*)cache, bs, (float*)q_out, qk_w, norm_first, v_from_k);
   else if (dim % 8 == 0 && dim <= 512 && ((dim >> 3) & ((dim >> 3) - 1)) == 0 && stride % 8 == 0 &&
            rot_dims % (interleaved ? 8 : 16) == 0 &&
            (((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)cache | (uintptr_t)bias | (uintptr_t)cos_sin) & 15) == 0) {
@@ -749,23 +800,23 @@ void sm_qkv_rope_cache(const void* qkv, int64_t stride, const float* bias, const
     const dim3 vgrid(T, std::max(1, std::min(per_tok_v, 4096 / T)));
     hipLaunchKernelGGL(qkv_rope_cache_vec_kernel, vgrid, dim3(NT), 0, stream, (const bf16_t*)qkv, stride, bias, positions,
                        cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit, eps, v_first, v_mode, lam, slots,
-                       (bf16_t*)cache, bs, (bf16_t*)q_out, qk_w);
+                       (bf16_t*)cache, bs, (bf16_t*)q_out, qk_w, norm_first, v_from_k);
   } else
     hipLaunchKernelGGL((qkv_rope_cache_kernel<bf16_t>), grid, dim3(NT), 0, stream, (const bf16_t*)qkv, stride, bias,
                        positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, interleaved, unit, eps, v_first, v_mode, lam,
-                       slots, (bf16_t*)cache, bs, (bf16_t*)q_out, qk_w);
+                       slots, (bf16_t*)cache, bs, (bf16_t*)q_out, qk_w, norm_first, v_from_k);
 }
 
 // Returns 0, or 1 when the sizes do not fit the kernel (vdim > 1024 or rows too wide for LDS).
 int sm_grouped_attention(const void* q, const void* cache, const int* tables, int W, int bs, const int* row_seq,
                          const int* row_len, float scale, int Hq, int Hkv, int dim, int vdim, int T, int QT,
                          const void* gate, int64_t gate_stride, void* out, int f32, const float* slopes, int chunk,
-                         const float* sinks, hipStream_t stream) {
+                         const float* sinks, int window, int keep, hipStream_t stream) {
   if (T == 0) return 0;
   const int vc = (vdim + 63) / 64;
 #define SM_GO(TYPE, VC)                                                                                          \
   return launch_attn<TYPE, VC>(q, cache, tables, W, bs, row_seq, row_len, scale, Hq, Hkv, dim, vdim, T, QT, gate, \
-                               gate_stride, out, slopes, chunk, sinks, stream)
+                               gate_stride, out, slopes, chunk, sinks, window, keep, stream)
   if (f32) {
     if (vc <= 1) SM_GO(float, 1);
     if (vc <= 2) SM_GO(float, 2);
@@ -790,7 +841,7 @@ int sm_grouped_attention_mfma(const void* q, const void* cache, const int* table
                               int n_items, const int* row_len, float scale, int Hq, int Hkv, int dim, int vdim,
                               const void* gate, int64_t gate_stride, void* out, int nsplit, int split_keys,
                               float* part_o, float* part_ml, int rb, const float* slopes, int chunk,
-                              const float* sinks, hipStream_t stream) {
+                              const float* sinks, int window, int keep, hipStream_t stream) {
   if (n_items == 0) return 0;
   const int nks = (dim + 31) / 32, ncb = (vdim + 15) / 16;
   if (Hq / Hkv > 64 || nks > 8 || ncb > 16 || (rb != 1 && rb != 2) || (nsplit > 1 && rb != 1) || bs % 8) return 1;
@@ -800,7 +851,7 @@ int sm_grouped_attention_mfma(const void* q, const void* cache, const int* table
   hipLaunchKernelGGL((grouped_attention_mfma_kernel<NKS, NCB, RB>), grid, dim3(NT), 0, stream, (const bf16_t*)q,   \
                      (const bf16_t*)cache, tables, W, bs, items, row_len, scale, Hq, Hkv, dim, vdim,               \
                      (const bf16_t*)gate, gate_stride, (bf16_t*)out, split_keys, part_o, part_ml, slopes, chunk, \
-                     sinks)
+                     sinks, window, keep)
 #define SM_GO2(NKS, NCB) \
   if (rb == 2) SM_GO(NKS, NCB, 2); \
   else SM_GO(NKS, NCB, 1)

@@ -1,9 +1,11 @@
 // Latent attention of any size over a paged latent cache (one row [latent R | rotated key dr]
 // per token, shared by all heads).
 //
-// latent_rope_cache: rotate the query's rotary part (rotate-half pairs over the first
-//   rot_dims dimensions, angles from an fp32 cos/sin table) into the absorbed query, RMS-norm the
-//   latent with its plain weight, rotate the shared key part and write the cache row.
+// latent_rope_cache: rotate the query's rotary part (pairs (i, i + rot_dims/2) or (2i, 2i+1) over
+//   the first rot_dims dimensions, angles from an fp32 cos/sin table) into the absorbed query, RMS-norm
+//   the latent with its plain weight, rotate the shared key part and write the cache row. A layer
+//   that reads another layer's cache passes no kv and rotates its queries only.
+// All attention forms take an optional gate [T, H]: head h's result times sigmoid(gate[t, h]).
 // latent_attention: one workgroup = QT consecutive token rows x 4 heads (one wave per head).
 //   Keys stream through LDS in tiles of KT rows (fp32) shared by all 4 x QT (row, head) pairs;
 //   a lane scores one key (dot over R + dr from LDS), the wave keeps an online softmax per pair,
@@ -23,22 +25,29 @@ __global__ __launch_bounds__(NT) void latent_rope_cache_kernel(
     const T* __restrict__ q, int64_t q_stride, const T* __restrict__ kv, int64_t kv_stride,
     const T* __restrict__ norm_w, float eps, const int64_t* __restrict__ positions,
     const float* __restrict__ cos_sin, int H, int dn, int dr, int rot_dims, int R,
-    const int64_t* __restrict__ slots, T* __restrict__ cache, T* __restrict__ q_abs) {
+    const int64_t* __restrict__ slots, T* __restrict__ cache, T* __restrict__ q_abs, int interleaved) {
   __shared__ float red[NT / 64];
   const int64_t t = blockIdx.x;
   const int half = rot_dims >> 1;
   const float* cs = cos_sin + positions[t] * rot_dims;  // [cos(half) | sin(half)]
   const int Dk = R + dr;
+  // element i of a rotated vector at src
+  auto rot = [&](const T* src, int i) {
+    if (i >= rot_dims) return ld(src + i);
+    if (interleaved) {
+      const int f = i >> 1;
+      return (i & 1) ? ld(src + i) * cs[f] + ld(src + i - 1) * cs[half + f]
+                     : ld(src + i) * cs[f] - ld(src + i + 1) * cs[half + f];
+    }
+    return i < half ? ld(src + i) * cs[i] - ld(src + i + half) * cs[half + i]
+                    : ld(src + i) * cs[i - half] + ld(src + i - half) * cs[i];
+  };
   // query: rotary part of every head -> q_abs[t, h, R + i]
   for (int e = threadIdx.x; e < H * dr; e += NT) {
     const int h = e / dr, i = e - h * dr;
-    const T* src = q + t * q_stride + (int64_t)h * (dn + dr) + dn;
-    float v;
-    if (i < half) v = ld(src + i) * cs[i] - ld(src + i + half) * cs[half + i];
-    else if (i < rot_dims) v = ld(src + i) * cs[i - half] + ld(src + i - half) * cs[i];
-    else v = ld(src + i);
-    st(q_abs + (t * H + h) * Dk + R + i, v);
+    st(q_abs + (t * H + h) * Dk + R + i, rot(q + t * q_stride + (int64_t)h * (dn + dr) + dn, i));
   }
+  if (kv == nullptr) return;
   // latent: RMS norm with a plain weight
   const T* kr = kv + t * kv_stride;
   float ss = 0.f;
@@ -52,14 +61,7 @@ __global__ __launch_bounds__(NT) void latent_rope_cache_kernel(
   const float inv = 1.f / sqrtf(ss / (float)R + eps);
   T* row = cache + slot * Dk;
   for (int c = threadIdx.x; c < R; c += NT) st(row + c, ld(kr + c) * inv * ld(norm_w + c));
-  const T* src = kr + R;
-  for (int i = threadIdx.x; i < dr; i += NT) {
-    float v;
-    if (i < half) v = ld(src + i) * cs[i] - ld(src + i + half) * cs[half + i];
-    else if (i < rot_dims) v = ld(src + i) * cs[i - half] + ld(src + i - half) * cs[i];
-    else v = ld(src + i);
-    st(row + R + i, v);
-  }
+  for (int i = threadIdx.x; i < dr; i += NT) st(row + R + i, rot(kr + R, i));
 }
 
 // RC = ceil(R / 64) output columns per lane; QT token rows per workgroup.
@@ -67,7 +69,7 @@ template <typename T, int RC, int QT>
 __global__ __launch_bounds__(NT) void latent_attention_kernel(
     const T* __restrict__ q_abs, const T* __restrict__ cache, const int* __restrict__ tables, int W, int bs,
     const int* __restrict__ row_seq, const int* __restrict__ row_len, float scale, int H, int R, int Dk, int KT,
-    int T_rows, T* __restrict__ out) {
+    int T_rows, T* __restrict__ out, const T* __restrict__ gate, int64_t gate_stride) {
   extern __shared__ float lds[];
   const int KS = Dk + 1;                 // key row stride in LDS (odd: lanes hit distinct banks)
   float* sK = lds;                       // [KT][KS]
@@ -167,7 +169,8 @@ __global__ __launch_bounds__(NT) void latent_attention_kernel(
       if (!act[r]) continue;
       done[r] = true;
       if (!head_ok) continue;
-      const float inv = 1.f / l[r];
+      float inv = 1.f / l[r];
+      if (gate) inv *= 1.f / (1.f + expf(-ld(gate + (int64_t)(t0 + r) * gate_stride + h)));
 #pragma unroll
       for (int c = 0; c < RC; ++c) {
         const int col = lane + 64 * c;
@@ -196,7 +199,8 @@ template <int NKS, int NCB>
 __global__ __launch_bounds__(NT) void latent_attention_mfma_kernel(
     const bf16_t* __restrict__ q_abs, const bf16_t* __restrict__ cache, const int* __restrict__ tables, int W, int bs,
     const int* __restrict__ items, const int* __restrict__ row_len, float scale, int H, int R, int Dk,
-    bf16_t* __restrict__ out, int split_keys, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    bf16_t* __restrict__ out, int split_keys, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const bf16_t* __restrict__ gate, int64_t gate_stride) {
   constexpr int DkP = 32 * NKS, RP = 16 * NCB;
   constexpr int KS = DkP + 8, VS = MKT + 8, PS = MKT + 8;  // LDS row strides (bf16), 16-byte multiples
   // The weights P live in the key tile's space once the scores are done (one more barrier per
@@ -372,10 +376,12 @@ __global__ __launch_bounds__(NT) void latent_attention_mfma_kernel(
     const int row = wave * 16 + kq * 4 + r;
     if (row >= ntok * H) continue;
     const int64_t base = ((int64_t)(tok0 + row / H) * H + row % H) * R;
+    float w = inv[r];
+    if (gate) w *= 1.f / (1.f + expf(-ld(gate + (int64_t)(tok0 + row / H) * gate_stride + row % H)));
 #pragma unroll
     for (int n = 0; n < NCB; ++n) {
       const int col = n * 16 + r16;
-      if (col < R) st(out + base + col, o[n][r] * inv[r]);
+      if (col < R) st(out + base + col, o[n][r] * w);
     }
   }
 }
@@ -384,7 +390,9 @@ __global__ __launch_bounds__(NT) void latent_attention_mfma_kernel(
 __global__ __launch_bounds__(NT) void latent_attention_merge_kernel(const int* __restrict__ items, int nsplit,
                                                                    const float* __restrict__ part_o,
                                                                    const float* __restrict__ part_ml, int H, int R,
-                                                                   bf16_t* __restrict__ out) {
+                                                                   bf16_t* __restrict__ out,
+                                                                   const bf16_t* __restrict__ gate,
+                                                                   int64_t gate_stride) {
   const int item = blockIdx.x, row = blockIdx.y;
   const int tok0 = items[item * 3 + 1], ntok = items[item * 3 + 2];
   if (row >= ntok * H) return;
@@ -396,6 +404,7 @@ __global__ __launch_bounds__(NT) void latent_attention_merge_kernel(const int* _
     L += expf(ml[0] - M) * ml[1];  // an empty range has m = -inf, l = 0
   }
   const int64_t obase = ((int64_t)(tok0 + row / H) * H + row % H) * R;
+  if (gate) L *= 1.f + expf(-ld(gate + (int64_t)(tok0 + row / H) * gate_stride + row % H));  // a / L * sigmoid
   for (int c = threadIdx.x; c < R; c += NT) {
     float a = 0.f;
     for (int y = 0; y < nsplit; ++y) {
@@ -409,7 +418,7 @@ __global__ __launch_bounds__(NT) void latent_attention_merge_kernel(const int* _
 template <typename T, int RC>
 int launch_attn(const void* q_abs, const void* cache, const int* tables, int W, int bs, const int* row_seq,
                 const int* row_len, float scale, int H, int R, int Dk, int T_rows, int QT, void* out,
-                hipStream_t stream) {
+                const void* gate, int64_t gate_stride, hipStream_t stream) {
   // key tile: as many of 64 / 32 / 16 rows as fit beside the queries in 128 KB of LDS
   int KT = 64;
   while (KT > 16 && ((size_t)KT * (Dk + 1) + (size_t)QT * 4 * Dk) * 4 > 128 * 1024) KT >>= 1;
@@ -419,7 +428,7 @@ int launch_attn(const void* q_abs, const void* cache, const int* tables, int W, 
   auto go = [&](auto kern) {
     if (lds > 64 * 1024) (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(kern, grid, dim3(NT), lds, stream, (const T*)q_abs, (const T*)cache, tables, W, bs, row_seq,
-                       row_len, scale, H, R, Dk, KT, T_rows, (T*)out);
+                       row_len, scale, H, R, Dk, KT, T_rows, (T*)out, (const T*)gate, gate_stride);
   };
   if (QT == 4) go(latent_attention_kernel<T, RC, 4>);
   else go(latent_attention_kernel<T, RC, 1>);
@@ -432,26 +441,26 @@ extern "C" {
 
 void sm_latent_rope_cache(const void* q, int64_t q_stride, const void* kv, int64_t kv_stride, const void* norm_w,
                           float eps, const int64_t* positions, const float* cos_sin, int H, int dn, int dr,
-                          int rot_dims, int R, const int64_t* slots, void* cache, void* q_abs, int T, int f32,
-                          hipStream_t stream) {
+                          int rot_dims, int R, const int64_t* slots, void* cache, void* q_abs, int interleaved, int T,
+                          int f32, hipStream_t stream) {
   if (T == 0) return;
   if (f32)
     hipLaunchKernelGGL((latent_rope_cache_kernel<float>), dim3(T), dim3(NT), 0, stream, (const float*)q, q_stride,
                        (const float*)kv, kv_stride, (const float*)norm_w, eps, positions, cos_sin, H, dn, dr,
-                       rot_dims, R, slots, (float*)cache, (float*)q_abs);
+                       rot_dims, R, slots, (float*)cache, (float*)q_abs, interleaved);
   else
     hipLaunchKernelGGL((latent_rope_cache_kernel<bf16_t>), dim3(T), dim3(NT), 0, stream, (const bf16_t*)q, q_stride,
                        (const bf16_t*)kv, kv_stride, (const bf16_t*)norm_w, eps, positions, cos_sin, H, dn, dr,
-                       rot_dims, R, slots, (bf16_t*)cache, (bf16_t*)q_abs);
+                       rot_dims, R, slots, (bf16_t*)cache, (bf16_t*)q_abs, interleaved);
 }
 
 // Returns 0, or 1 when the sizes do not fit the kernel (R > 1024 or rows too wide for LDS).
 int sm_latent_attention(const void* q_abs, const void* cache, const int* tables, int W, int bs, const int* row_seq,
                         const int* row_len, float scale, int H, int R, int Dk, int T, int QT, void* out, int f32,
-                        hipStream_t stream) {
+                        const void* gate, int64_t gate_stride, hipStream_t stream) {
   if (T == 0) return 0;
   const int rc = (R + 63) / 64;
-#define SM_GO(TYPE, RC) return launch_attn<TYPE, RC>(q_abs, cache, tables, W, bs, row_seq, row_len, scale, H, R, Dk, T, QT, out, stream)
+#define SM_GO(TYPE, RC) return launch_attn<TYPE, RC>(q_abs, cache, tables, W, bs, row_seq, row_len, scale, H, R, Dk, T, QT, out, gate, gate_stride, stream)
   if (f32) {
     if (rc <= 1) SM_GO(float, 1);
     if (rc <= 2) SM_GO(float, 2);
@@ -476,7 +485,8 @@ int sm_latent_attention(const void* q_abs, const void* cache, const int* tables,
 // Returns 0, or 1 when the sizes are outside the compiled forms (Dk > 576, R > 512, H > 64).
 int sm_latent_attention_mfma(const void* q_abs, const void* cache, const int* tables, int W, int bs, const int* items,
                              int n_items, const int* row_len, float scale, int H, int R, int Dk, void* out,
-                             int nsplit, int split_keys, float* part_o, float* part_ml, hipStream_t stream) {
+                             int nsplit, int split_keys, float* part_o, float* part_ml, const void* gate,
+                             int64_t gate_stride, hipStream_t stream) {
   if (n_items == 0) return 0;
   const int nks = (Dk + 31) / 32, ncb = (R + 15) / 16;
   if (H > 64 || nks > 18 || ncb > 32) return 1;
@@ -484,7 +494,7 @@ int sm_latent_attention_mfma(const void* q_abs, const void* cache, const int* ta
 #define SM_GO(NKS, NCB)                                                                                            \
   hipLaunchKernelGGL((latent_attention_mfma_kernel<NKS, NCB>), grid, dim3(NT), 0, stream, (const bf16_t*)q_abs,     \
                      (const bf16_t*)cache, tables, W, bs, items, row_len, scale, H, R, Dk, (bf16_t*)out, split_keys, \
-                     part_o, part_ml)
+                     part_o, part_ml, nsplit > 1 ? nullptr : (const bf16_t*)gate, gate_stride)
   if (nks <= 3 && ncb <= 4) SM_GO(3, 4);
   else if (nks <= 6 && ncb <= 8) SM_GO(6, 8);
   else if (nks <= 10 && ncb <= 16) SM_GO(10, 16);
@@ -492,7 +502,7 @@ int sm_latent_attention_mfma(const void* q_abs, const void* cache, const int* ta
 #undef SM_GO
   if (nsplit > 1)
     hipLaunchKernelGGL(latent_attention_merge_kernel, dim3(n_items, 64), dim3(NT), 0, stream, items, nsplit, part_o,
-                       part_ml, H, R, (bf16_t*)out);
+                       part_ml, H, R, (bf16_t*)out, (const bf16_t*)gate, gate_stride);
   return 0;
 }
 

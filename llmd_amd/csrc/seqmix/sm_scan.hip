@@ -3,6 +3,7 @@
 //
 // causal_conv_silu : per-channel short convolution + SiLU; the last taps-1 inputs of a sequence
 //                    are its convolution state (a second small kernel rolls it forward).
+// input_conv       : h + conv(h), the same convolution without bias and activation, added to its input.
 // selective_scan   : S[c,n] <- exp(dt_c A[c,n]) S[c,n] + dt_c x_c B_n; y_c = sum_n S[c,n] C_n + D_c x_c;
 //                    y * silu(z). A channel's states sit in neighbouring lanes (groups of NL), the
 //                    sum over n is a shuffle reduction; softplus, exp and the state are fp32.
@@ -64,6 +65,34 @@ __global__ __launch_bounds__(NT) void conv_state_kernel(const T* __restrict__ xz
     else if (init) v = ld(st_ + (int64_t)(taps - 1 + pp) * C + c);
     st(st_ + (int64_t)j * C + c, v);
   }
+}
+
+// out = h + conv(h): one thread per (token, channel). The token's earlier inputs come from the run
+// itself, from the sequence's state (its last taps - 1 inputs before this step) or are zero.
+template <typename T>
+__global__ __launch_bounds__(NT) void input_conv_kernel(const T* __restrict__ h, int C, const T* __restrict__ w,
+                                                       int taps, const T* __restrict__ state,
+                                                       const int* __restrict__ row_seq,
+                                                       const int* __restrict__ seq_start,
+                                                       const int* __restrict__ seq_slot,
+                                                       const int* __restrict__ seq_init, T* __restrict__ out) {
+  const int c = blockIdx.y * NT + threadIdx.x;
+  const int64_t t = blockIdx.x;
+  if (c >= C) return;
+  const int s = row_seq[t];
+  const int p = (int)t - seq_start[s];  // place in the run
+  const bool init = seq_init[s] != 0;
+  const T* st_ = state + (int64_t)seq_slot[s] * (taps - 1) * C;
+  const float x = ld(h + t * C + c);
+  float a = x + ld(w + (int64_t)c * taps + taps - 1) * x;
+  for (int j = 0; j < taps - 1; ++j) {
+    const int pp = p - (taps - 1 - j);
+    float v = 0.f;
+    if (pp >= 0) v = ld(h + (t - (taps - 1 - j)) * C + c);
+    else if (init) v = ld(st_ + (int64_t)(taps - 1 + pp) * C + c);
+    a += ld(w + (int64_t)c * taps + j) * v;
+  }
+  st(out + t * C + c, a);
 }
 
 // NL lanes per channel (power of two <= 64), SPL states per lane.
@@ -302,6 +331,26 @@ void sm_causal_conv_silu(const void* xz, int64_t xz_stride, int C, const void* w
                        (bf16_t*)out, seg);
     if (taps > 1)
       hipLaunchKernelGGL((conv_state_kernel<bf16_t>), g2, dim3(NT), 0, stream, (const bf16_t*)xz, xz_stride, C, taps,
+                         (bf16_t*)state, seq_start, seq_slot, seq_init);
+  }
+}
+
+void sm_input_conv(const void* h, int C, const void* w, int taps, void* state, const int* row_seq,
+                   const int* seq_start, const int* seq_slot, const int* seq_init, void* out, int T, int nseq, int f32,
+                   hipStream_t stream) {
+  if (nseq == 0 || T == 0) return;
+  const dim3 g1(T, (C + NT - 1) / NT), g2((C + NT - 1) / NT, nseq);
+  if (f32) {
+    hipLaunchKernelGGL((input_conv_kernel<float>), g1, dim3(NT), 0, stream, (const float*)h, C, (const float*)w, taps,
+                       (const float*)state, row_seq, seq_start, seq_slot, seq_init, (float*)out);
+    if (taps > 1)
+      hipLaunchKernelGGL((conv_state_kernel<float>), g2, dim3(NT), 0, stream, (const float*)h, (int64_t)C, C, taps,
+                         (float*)state, seq_start, seq_slot, seq_init);
+  } else {
+    hipLaunchKernelGGL((input_conv_kernel<bf16_t>), g1, dim3(NT), 0, stream, (const bf16_t*)h, C, (const bf16_t*)w,
+                       taps, (const bf16_t*)state, row_seq, seq_start, seq_slot, seq_init, (bf16_t*)out);
+    if (taps > 1)
+      hipLaunchKernelGGL((conv_state_kernel<bf16_t>), g2, dim3(NT), 0, stream, (const bf16_t*)h, (int64_t)C, C, taps,
                          (bf16_t*)state, seq_start, seq_slot, seq_init);
   }
 }
