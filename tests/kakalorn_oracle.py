@@ -197,3 +197,65 @@ def forward(cfg, W, tokens, layers_out=None):
         if layers_out is not None:
             layers_out.append(x.clone())
     return rms_norm(x, W["final.norm"], eps) @ W["head"].to(F64).T
+
+
+def random_weights(cfg, seed=0, dtype=torch.float32):
+    """Random tensors with the design's names and shapes (std chosen so that nothing saturates)."""
+    g = torch.Generator().manual_seed(seed)
+    d, V = cfg["width"], cfg["vocab"]
+    taps = cfg["canon"]["taps"]
+    W = {}
+
+    def mat(name, *shape, std=None):
+        std = std if std is not None else 1.0 / math.sqrt(shape[-1])
+        W[name] = (torch.randn(*shape, generator=g) * std).to(dtype)
+
+    def vec(name, n, mean=1.0, std=0.1):
+        W[name] = (mean + torch.randn(n, generator=g) * std).to(dtype)
+
+    mat("embed", V, d, std=1.0)
+    for i, spec in enumerate(cfg["layers"]):
+        pre, m = f"l{i}.", spec["mixer"]
+        vec(pre + "norm1", d)
+        vec(pre + "norm1b", d)
+        mat(pre + "canon1", d, taps, std=0.4)
+        mp = pre + "mix."
+        if spec["type"] == "attention":
+            H, G, dim = m["heads"], m["kv_heads"], m["dim"]
+            mat(mp + "q", H * dim, d)
+            mat(mp + "k", G * dim, d)
+            vec(mp + "q.b", H * dim, mean=0.0, std=0.3)
+            vec(mp + "k.b", G * dim, mean=0.0, std=0.3)
+            vec(mp + "q.norm", dim, std=0.3)
+            vec(mp + "k.norm", dim, std=0.3)
+            vec(mp + "sink", H, mean=0.0, std=1.0)
+            mat(mp + "o", d, H * dim)
+        elif spec["type"] == "hgrn2":
+            H, dim, dv = m["heads"], m["dim"], m["vdim"]
+            mat(mp + "q", H * dim, d)
+            mat(mp + "f", H * dim, d)
+            vec(mp + "f.b", H * dim, mean=0.5, std=1.0)
+            W[mp + "lower"] = torch.rand(H * dim, generator=g).to(dtype)
+            mat(mp + "v", H * dv, d)
+            vec(mp + "norm", dv)
+            mat(mp + "o", d, H * dv)
+        else:
+            H, dim, dr, dv, R, Q = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"], m["q_rank"]
+            mat(mp + "dq", Q, d)
+            vec(mp + "dq.norm", Q)
+            mat(mp + "uq", H * (dim + dr), Q)
+            if m.get("kv_from") is None:
+                mat(mp + "dkv", R + dr, d)
+                vec(mp + "dkv.norm", R)
+            mat(mp + "uk", H * dim, R)
+            mat(mp + "uv", H * dv, R)
+            mat(mp + "g", H, d)
+            mat(mp + "o", d, H * dv)
+        if spec.get("mlp"):
+            vec(pre + "norm2", d)
+            vec(pre + "norm2b", d)
+            mat(pre + "mlp.up", spec["mlp"]["ff"], d)
+            mat(pre + "mlp.down", d, spec["mlp"]["ff"])
+    vec("final.norm", d)
+    mat("head", V, d)
+    return W
