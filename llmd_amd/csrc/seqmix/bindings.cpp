@@ -25,7 +25,7 @@ void sm_embed_norm(const int64_t*, const void*, int64_t, const void*, float, flo
 void sm_rms_norm_rows(const void*, int64_t, const void*, float, void*, int, int, int, hipStream_t);
 void sm_relu2(const void*, void*, int64_t, int, hipStream_t);
 void sm_input_conv(const void*, int, const void*, int, void*, const int*, const int*, const int*, const int*, void*,
-                   int, int, int, hipStream_t);
+                   int, int, int, int, hipStream_t);
 int sm_hgrn2_scan(const void*, int64_t, int, int, int, const float*, const float*, const void*, float, float*,
                   const int*, const int*, const int*, void*, float*, float*, float*, float*, int, int, int,
                   hipStream_t);
@@ -743,7 +743,7 @@ void relu2(Tensor z, Tensor out) {
 }
 
 void input_conv(Tensor h, Tensor w, Tensor state, Tensor row_seq, Tensor seq_start, Tensor seq_slot, Tensor seq_init,
-                Tensor out) {
+                int64_t max_q, Tensor out) {
   const c10::hip::OptionalHIPGuard g(dev_of(h));
   TORCH_CHECK(h.is_cuda() && act_ok(h) && h.dim() == 2 && h.is_contiguous(), "h [T, C]");
   const int64_t T = h.size(0), C = h.size(1);
@@ -756,11 +756,11 @@ void input_conv(Tensor h, Tensor w, Tensor state, Tensor row_seq, Tensor seq_sta
                   (taps == 1 || state.size(1) == taps - 1), "conv state [slots, taps-1, C]");
   check_seq(seq_start, seq_slot, seq_init, state.size(0));
   CHECK_I32(row_seq);
-  TORCH_CHECK(row_seq.numel() == T && seq_slot.numel() <= 65535, "row_seq [T]");
+  TORCH_CHECK(row_seq.numel() == T && seq_slot.numel() <= 65535 && max_q >= 1 && max_q <= T, "row_seq [T], longest run");
   TORCH_CHECK(out.is_contiguous() && out.numel() == T * C, "out [T, C]");
   sm_input_conv(h.data_ptr(), C, w.data_ptr(), taps, state.data_ptr(), row_seq.data_ptr<int>(),
                 seq_start.data_ptr<int>(), seq_slot.data_ptr<int>(), seq_init.data_ptr<int>(), out.data_ptr(), T,
-                seq_slot.numel(), is_f32(h), cur());
+                seq_slot.numel(), max_q, is_f32(h), cur());
 }
 
 void hgrn2_scan(Tensor p, int64_t H, int64_t dk, int64_t dv, Tensor f_bias, Tensor lower, Tensor norm_w, double eps,

@@ -231,6 +231,24 @@ __global__ __launch_bounds__(NT) void rms_norm_rows_kernel(const T* __restrict__
   for (int c = lane; c < n; c += 64) st(out + row * n + c, ld(yr + c) * inv * ld(w + c));
 }
 
+// the same with a workgroup per row: long rows of small steps
+template <typename T>
+__global__ __launch_bounds__(NT) void rms_norm_row_block_kernel(const T* __restrict__ y, int64_t y_stride,
+                                                               const T* __restrict__ w, float eps,
+                                                               T* __restrict__ out, int n) {
+  __shared__ float red[NT / 64];
+  const int64_t row = blockIdx.x;
+  const T* yr = y + row * y_stride;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < n; c += NT) {
+    const float v = ld(yr + c);
+    ss += v * v;
+  }
+  ss = block_sum<NT>(ss, red);
+  const float inv = 1.f / sqrtf(ss / (float)n + eps);
+  for (int c = threadIdx.x; c < n; c += NT) st(out + row * n + c, ld(yr + c) * inv * ld(w + c));
+}
+
 template <typename T>
 __global__ __launch_bounds__(NT) void relu2_kernel(const T* __restrict__ z, T* __restrict__ out, int64_t n) {
   const int64_t i = (int64_t)blockIdx.x * NT + threadIdx.x;
@@ -272,6 +290,15 @@ void sm_embed_norm(const int64_t* ids, const void* table, int64_t V, const void*
 void sm_rms_norm_rows(const void* y, int64_t y_stride, const void* w, float eps, void* out, int rows, int n, int f32,
                       hipStream_t stream) {
   if (rows == 0) return;
+  if (n >= 512 && rows <= 16384) {  // a wave would walk a long row alone
+    if (f32)
+      hipLaunchKernelGGL((rms_norm_row_block_kernel<float>), dim3(rows), dim3(NT), 0, stream, (const float*)y, y_stride,
+                         (const float*)w, eps, (float*)out, n);
+    else
+      hipLaunchKernelGGL((rms_norm_row_block_kernel<bf16_t>), dim3(rows), dim3(NT), 0, stream, (const bf16_t*)y,
+                         y_stride, (const bf16_t*)w, eps, (bf16_t*)out, n);
+    return;
+  }
   const dim3 grid((rows + NT / 64 - 1) / (NT / 64));
   if (f32)
     hipLaunchKernelGGL((rms_norm_rows_kernel<float>), grid, dim3(NT), 0, stream, (const float*)y, y_stride,

@@ -51,11 +51,12 @@ template <typename T>
 __global__ __launch_bounds__(NT) void conv_state_kernel(const T* __restrict__ xz, int64_t xz_stride, int C, int taps,
                                                        T* __restrict__ state, const int* __restrict__ seq_start,
                                                        const int* __restrict__ seq_slot,
-                                                       const int* __restrict__ seq_init) {
+                                                       const int* __restrict__ seq_init, int skip_single = 0) {
   const int c = blockIdx.x * NT + threadIdx.x;
   const int s = blockIdx.y;
   if (c >= C) return;
   const int lo = seq_start[s], len = seq_start[s + 1] - lo;
+  if (len <= 0 || (skip_single && len == 1)) return;  // a single token's roll was done where it was computed
   const bool init = seq_init[s] != 0;
   T* st_ = state + (int64_t)seq_slot[s] * (taps - 1) * C;
   for (int j = 0; j < taps - 1; ++j) {  // ascending j reads old entries j + len > j not yet rewritten
@@ -71,7 +72,7 @@ __global__ __launch_bounds__(NT) void conv_state_kernel(const T* __restrict__ xz
 // itself, from the sequence's state (its last taps - 1 inputs before this step) or are zero.
 template <typename T>
 __global__ __launch_bounds__(NT) void input_conv_kernel(const T* __restrict__ h, int C, const T* __restrict__ w,
-                                                       int taps, const T* __restrict__ state,
+                                                       int taps, T* state,
                                                        const int* __restrict__ row_seq,
                                                        const int* __restrict__ seq_start,
                                                        const int* __restrict__ seq_slot,
@@ -82,7 +83,7 @@ __global__ __launch_bounds__(NT) void input_conv_kernel(const T* __restrict__ h,
   const int s = row_seq[t];
   const int p = (int)t - seq_start[s];  // place in the run
   const bool init = seq_init[s] != 0;
-  const T* st_ = state + (int64_t)seq_slot[s] * (taps - 1) * C;
+  T* st_ = state + (int64_t)seq_slot[s] * (taps - 1) * C;
   const float x = ld(h + t * C + c);
   float a = x + ld(w + (int64_t)c * taps + taps - 1) * x;
   for (int j = 0; j < taps - 1; ++j) {
@@ -93,6 +94,72 @@ __global__ __launch_bounds__(NT) void input_conv_kernel(const T* __restrict__ h,
     a += ld(w + (int64_t)c * taps + j) * v;
   }
   st(out + t * C + c, a);
+  if (p == 0 && seq_start[s + 1] - seq_start[s] == 1) {
+    // a run of one token (a decode step): nobody else reads or writes this sequence's state, so it is
+    // rolled here; ascending j reads entry j + 1 before anything overwrites it
+    for (int j = 0; j < taps - 2; ++j) st(st_ + (int64_t)j * C + c, init ? ld(st_ + (int64_t)(j + 1) * C + c) : 0.f);
+    if (taps > 1) st(st_ + (int64_t)(taps - 2) * C + c, x);
+  }
+}
+
+// bf16 form with 16-byte accesses: a thread owns eight neighbouring channels of one token and keeps their
+// 8 x TAPS weights in registers (TAPS 16-byte loads: the weights of eight channels lie side by side).
+// C a multiple of 8, TAPS <= 8.
+constexpr int ICV_MAX_TAPS = 8;
+template <int TAPS>
+__global__ __launch_bounds__(NT) void input_conv_vec_kernel(const bf16_t* __restrict__ h, int C,
+                                                           const bf16_t* __restrict__ w, bf16_t* state,
+                                                           const int* __restrict__ row_seq,
+                                                           const int* __restrict__ seq_start,
+                                                           const int* __restrict__ seq_slot,
+                                                           const int* __restrict__ seq_init,
+                                                           bf16_t* __restrict__ out) {
+  const int c = (blockIdx.y * NT + threadIdx.x) * 8;
+  const int64_t t = blockIdx.x;
+  if (c >= C) return;
+  auto ld8 = [](const bf16_t* p, float* v) {
+    const uint4 q = *reinterpret_cast<const uint4*>(p);
+    v[0] = __uint_as_float(q.x << 16); v[1] = __uint_as_float(q.x & 0xffff0000u);
+    v[2] = __uint_as_float(q.y << 16); v[3] = __uint_as_float(q.y & 0xffff0000u);
+    v[4] = __uint_as_float(q.z << 16); v[5] = __uint_as_float(q.z & 0xffff0000u);
+    v[6] = __uint_as_float(q.w << 16); v[7] = __uint_as_float(q.w & 0xffff0000u);
+  };
+  float wr[8 * TAPS];  // channel i, tap j at i * TAPS + j
+#pragma unroll
+  for (int i = 0; i < TAPS; ++i) ld8(w + (int64_t)c * TAPS + 8 * i, wr + 8 * i);
+  const int s = row_seq[t];
+  const int lo = seq_start[s];
+  const int p = (int)t - lo;
+  const bool init = seq_init[s] != 0;
+  bf16_t* st_ = state + (int64_t)seq_slot[s] * (TAPS - 1) * C;
+  float x[8], a[8];
+  ld8(h + t * C + c, x);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) a[i] = x[i] + wr[i * TAPS + TAPS - 1] * x[i];
+#pragma unroll
+  for (int j = 0; j < TAPS - 1; ++j) {
+    const int pp = p - (TAPS - 1 - j);
+    float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (pp >= 0) ld8(h + (t - (TAPS - 1 - j)) * C + c, v);
+    else if (init) ld8(st_ + (int64_t)(TAPS - 1 + pp) * C + c, v);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a[i] += wr[i * TAPS + j] * v[i];
+  }
+  uint4 o;
+  auto pack = [](float lo_, float hi_) {
+    const __bf16 l16 = (__bf16)lo_, h16 = (__bf16)hi_;
+    return (uint32_t)__builtin_bit_cast(uint16_t, l16) | ((uint32_t)__builtin_bit_cast(uint16_t, h16) << 16);
+  };
+  o.x = pack(a[0], a[1]); o.y = pack(a[2], a[3]); o.z = pack(a[4], a[5]); o.w = pack(a[6], a[7]);
+  *reinterpret_cast<uint4*>(out + t * C + c) = o;
+  if (TAPS > 1 && p == 0 && seq_start[s + 1] - lo == 1) {  // a run of one token: its state is rolled here (see above)
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int j = 0; j < TAPS - 2; ++j)
+      *reinterpret_cast<uint4*>(st_ + (int64_t)j * C + c) =
+          init ? *reinterpret_cast<const uint4*>(st_ + (int64_t)(j + 1) * C + c) : zero;
+    *reinterpret_cast<uint4*>(st_ + (int64_t)(TAPS - 2) * C + c) = *reinterpret_cast<const uint4*>(h + t * C + c);
+  }
 }
 
 // NL lanes per channel (power of two <= 64), SPL states per lane.
@@ -335,23 +402,43 @@ void sm_causal_conv_silu(const void* xz, int64_t xz_stride, int C, const void* w
   }
 }
 
+// max_q: the longest run of the step; runs of one token roll their state in the first kernel, so a
+// decode-only step needs no second launch.
 void sm_input_conv(const void* h, int C, const void* w, int taps, void* state, const int* row_seq,
-                   const int* seq_start, const int* seq_slot, const int* seq_init, void* out, int T, int nseq, int f32,
-                   hipStream_t stream) {
+                   const int* seq_start, const int* seq_slot, const int* seq_init, void* out, int T, int nseq,
+                   int max_q, int f32, hipStream_t stream) {
   if (nseq == 0 || T == 0) return;
   const dim3 g1(T, (C + NT - 1) / NT), g2((C + NT - 1) / NT, nseq);
+  const bool roll = taps > 1 && max_q > 1;
+  if (!f32 && C % 8 == 0 && taps <= ICV_MAX_TAPS &&
+      (((uintptr_t)h | (uintptr_t)out | (uintptr_t)state | (uintptr_t)w) & 15) == 0) {
+    const dim3 gv(T, (C / 8 + NT - 1) / NT);
+#define SM_ICV(N)                                                                                                     \
+  case N:                                                                                                             \
+    hipLaunchKernelGGL(input_conv_vec_kernel<N>, gv, dim3(NT), 0, stream, (const bf16_t*)h, C, (const bf16_t*)w,      \
+                       (bf16_t*)state, row_seq, seq_start, seq_slot, seq_init, (bf16_t*)out);                        \
+    break
+    switch (taps) {
+      SM_ICV(1); SM_ICV(2); SM_ICV(3); SM_ICV(4); SM_ICV(5); SM_ICV(6); SM_ICV(7); SM_ICV(8);
+    }
+#undef SM_ICV
+    if (roll)
+      hipLaunchKernelGGL((conv_state_kernel<bf16_t>), g2, dim3(NT), 0, stream, (const bf16_t*)h, (int64_t)C, C, taps,
+                         (bf16_t*)state, seq_start, seq_slot, seq_init, 1);
+    return;
+  }
   if (f32) {
     hipLaunchKernelGGL((input_conv_kernel<float>), g1, dim3(NT), 0, stream, (const float*)h, C, (const float*)w, taps,
-                       (const float*)state, row_seq, seq_start, seq_slot, seq_init, (float*)out);
-    if (taps > 1)
+                       (float*)state, row_seq, seq_start, seq_slot, seq_init, (float*)out);
+    if (roll)
       hipLaunchKernelGGL((conv_state_kernel<float>), g2, dim3(NT), 0, stream, (const float*)h, (int64_t)C, C, taps,
-                         (float*)state, seq_start, seq_slot, seq_init);
+                         (float*)state, seq_start, seq_slot, seq_init, 1);
   } else {
     hipLaunchKernelGGL((input_conv_kernel<bf16_t>), g1, dim3(NT), 0, stream, (const bf16_t*)h, C, (const bf16_t*)w,
-                       taps, (const bf16_t*)state, row_seq, seq_start, seq_slot, seq_init, (bf16_t*)out);
-    if (taps > 1)
+                       taps, (bf16_t*)state, row_seq, seq_start, seq_slot, seq_init, (bf16_t*)out);
+    if (roll)
       hipLaunchKernelGGL((conv_state_kernel<bf16_t>), g2, dim3(NT), 0, stream, (const bf16_t*)h, (int64_t)C, C, taps,
-                         (bf16_t*)state, seq_start, seq_slot, seq_init);
+                         (bf16_t*)state, seq_start, seq_slot, seq_init, 1);
   }
 }
 

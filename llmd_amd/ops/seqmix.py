@@ -473,11 +473,12 @@ def rms_norm(y, w, eps: float):
 def input_conv(h, w, state, seq):
     """h + conv(h) per channel over each sequence's run: conv(h)_t = sum_j w[:, j] h_(t - taps + 1 + j),
     continuing from the sequence's last taps - 1 inputs in ``state`` [slots, taps - 1, C] (read when
-    seq_init is set, zeros otherwise; rolled forward to the run's end)."""
+    seq_init is set, zeros otherwise; rolled forward to the run's end). ``seq.max_q`` is the step's
+    longest run: a step of single tokens rolls the states in the same launch."""
     out = torch.empty_like(h)
     if not h.is_cuda:
         return ref.input_conv(h, w, state, seq.seq_start, seq.seq_slot, seq.seq_init, out)
-    native().input_conv(h, w, state, seq.row_seq, seq.seq_start, seq.seq_slot, seq.seq_init, out)
+    native().input_conv(h, w, state, seq.row_seq, seq.seq_start, seq.seq_slot, seq.seq_init, int(seq.max_q), out)
     return out
 
 

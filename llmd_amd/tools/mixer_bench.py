@@ -28,6 +28,18 @@ Two Zumizen stacks (post-norm residual, bigram embedding, experts whose score sc
                      bias, sink) beside a gated delta rule 16 heads / 8 q-k heads x 128 x 128; 128 experts,
                      8 chosen, ff 768 - beside ``negunex-moe`` (same attention and expert geometry)
 
+Four Kakalorn stacks (norms before and after every sublayer, a short convolution in front of every
+mixer, squared-ReLU feed-forwards):
+
+  kakalorn-window : width 4096, windowed attention 32 heads / 8 kv heads x 128 whose values are its keys
+                    (window 1024, 4 kept first tokens, learned sinks), dense ff 14336 - beside
+                    ``negunex-dense`` and Llama-3-8B layers (same heads and feed-forward size)
+  kakalorn-latent : width 2048, latent attention 16 heads x (128 + 64), value 128, latent 512, query
+                    latent 1536, head gates; dense ff 5632 - beside Mekusun's ``latent+moe`` (same attention)
+  kakalorn-hgrn2  : width 2048, HGRN2 32 heads x 64 (key) x 64 (value); dense ff 5632 - beside Mekusun's
+                    ``delta`` and ``zumizen-channel`` (same heads and sizes)
+  kakalorn-hybrid : width 2048, the three mixers in turn plus a latent layer that reads the other's cache
+
 Prefill: one prompt of ``--tokens`` tokens in one step. Decode: ``--batch`` sequences with that
 context, one token each. One JSON line with tokens/s and ms per layer for every entry.
 """
@@ -102,6 +114,39 @@ def _zumizen(kind: str):
                                      "layers": [layer] * n})
 
 
+def _kakalorn(kind: str):
+    from llmd_amd.engine.config import kakalorn_config
+
+    width = 4096 if kind == "window" else WIDTH
+    win = {"type": "attention",
+           "mixer": {"heads": 32, "kv_heads": 8 if kind == "window" else 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                     "mask": {"size": 1024, "keep_first": 4}, "rot": {"dims": 128, "base": 500000.0}},
+           "mlp": {"kind": "dense", "ff": 14336 if kind == "window" else 5632}}
+    lat = {"type": "latent_attention",
+           "mixer": {"heads": 16, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "q_rank": 1536,
+                     "scale": 192 ** -0.5,
+                     "rot": {"dims": 64, "base": 10000.0,
+                             "scaling": {"factor": 40.0, "original": 4096, "fast": 32.0, "slow": 1.0}}},
+           "mlp": {"kind": "dense", "ff": 5632}}
+    rec = {"type": "hgrn2", "mixer": {"heads": 32, "dim": 64, "vdim": 64}, "mlp": {"kind": "dense", "ff": 5632}}
+
+    def make(n):
+        if kind == "hybrid":
+            shared = json.loads(json.dumps(lat))
+            layers = []
+            for i in range(n):
+                layers.append([rec, lat, win, shared][i % 4])
+                if i % 4 == 3:
+                    layers[-1] = json.loads(json.dumps(shared))
+                    layers[-1]["mixer"]["kv_from"] = i - 2
+        else:
+            layers = [{"window": win, "latent": lat, "hgrn2": rec}[kind]] * n
+        return kakalorn_config({"architecture": "Kakalorn", "name": "kakalorn-" + kind, "width": width, "vocab": 32000,
+                                "norm": {"eps": 1e-6}, "canon": {"taps": 4}, "layers": layers})
+
+    return make
+
+
 def _runner(mc, tokens: int, batch: int, device: str):
     from llmd_amd.engine.config import EngineConfig
     from llmd_amd.engine.model_runner import ModelRunner
@@ -167,7 +212,11 @@ def run(tokens: int = 2048, batch: int = 32, n_layers: int = 4, reps: int = 5, d
             ("qwen3-30b-a3b layers", dataclasses.replace(get_model_config("qwen3-30b-a3b"), num_hidden_layers=n_layers,
                                                          vocab_size=32000, name="qwen3-30b-a3b-cut"), n_layers),
             ("zumizen-channel", _zumizen("channel")(n_layers), n_layers),
-            ("zumizen-parallel", _zumizen("parallel")(n_layers), n_layers)]
+            ("zumizen-parallel", _zumizen("parallel")(n_layers), n_layers),
+            ("kakalorn-window", _kakalorn("window")(n_layers), n_layers),
+            ("kakalorn-latent", _kakalorn("latent")(n_layers), n_layers),
+            ("kakalorn-hgrn2", _kakalorn("hgrn2")(n_layers), n_layers),
+            ("kakalorn-hybrid", _kakalorn("hybrid")(n_layers), n_layers)]
     for name, mc, L in todo:
         if only and not any(name.startswith(o) for o in only.split(",")):
             continue

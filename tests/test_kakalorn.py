@@ -205,11 +205,11 @@ def test_squared_relu(device, dtype, shape):
 
 @pytest.mark.parametrize("device,dtype", ATT_DTYPES)
 @pytest.mark.parametrize("taps", [1, 2, 4, 7])
-@pytest.mark.parametrize("C", [40, 300])
+@pytest.mark.parametrize("C", [40, 300, 4104])
 def test_input_convolution_continues_each_sequence(device, dtype, taps, C):
-    """Two sequences in portions over three steps (one token, two tokens, fewer tokens than taps), their
-    slots swapped against the order of the step; a third sequence takes over a used slot and starts
-    from zeros again."""
+    """Two sequences in portions over several steps (one token, two tokens, fewer tokens than taps, a
+    step of single tokens only), their slots swapped against the order of the step; a third sequence
+    takes over a used slot and starts from zeros again."""
     g = torch.Generator().manual_seed(taps * C)
     w = (torch.randn(C, taps, generator=g) * 0.5).to(dtype)
     ha, hb, hc = (torch.randn(n, C, generator=g).to(dtype) for n in (12, 6, 4))
@@ -217,7 +217,8 @@ def test_input_convolution_continues_each_sequence(device, dtype, taps, C):
     state = torch.randn(3, max(taps - 1, 1), C, generator=g).to(dtype).to(device)      # slots hold something old
     got = {"a": [], "b": [], "c": []}
     steps = [[("a", ha[:1], 2, 0), ("b", hb[:2], 0, 0)], [("b", hb[2:3], 0, 1), ("a", ha[1:3], 2, 1)],
-             [("a", ha[3:4], 2, 1), ("b", hb[3:], 0, 1)], [("a", ha[4:], 2, 1), ("c", hc, 0, 0)]]
+             [("a", ha[3:4], 2, 1), ("b", hb[3:4], 0, 1)], [("b", hb[4:5], 0, 1), ("a", ha[4:5], 2, 1)],
+             [("a", ha[5:6], 2, 1), ("b", hb[5:], 0, 1)], [("a", ha[6:], 2, 1), ("c", hc, 0, 0)]]
     for step in steps:
         h = torch.cat([x for _, x, _, _ in step]).to(device)
         seq = _seq(device, [x.shape[0] for _, x, _, _ in step], [s for _, _, s, _ in step], [i for _, _, _, i in step])
