@@ -27,8 +27,8 @@ void sm_relu2(const void*, void*, int64_t, int, hipStream_t);
 void sm_input_conv(const void*, int, const void*, int, void*, const int*, const int*, const int*, const int*, void*,
                    int, int, int, int, hipStream_t);
 int sm_hgrn2_scan(const void*, int64_t, int, int, int, const float*, const float*, const void*, float, float*,
-                  const int*, const int*, const int*, void*, float*, float*, float*, float*, int, int, int,
-                  hipStream_t);
+                  const int*, const int*, const int*, void*, float*, float*, float*, float*, int, int, int, int,
+                  const int*, const int*, const int*, const int*, const int*, float*, float*, hipStream_t);
 void sm_causal_conv_silu(const void*, int64_t, int, const void*, const void*, int, void*, const int*, const int*,
                          const int*, void*, int, int, int, hipStream_t);
 int sm_selective_scan(const void*, const void*, const void*, const float*, const void*, int64_t, int, int, const void*,
@@ -763,8 +763,11 @@ void input_conv(Tensor h, Tensor w, Tensor state, Tensor row_seq, Tensor seq_sta
                 seq_slot.numel(), max_q, is_f32(h), cur());
 }
 
+// chunks: int32 [4 nc + 1 + nseq + 1] = [chunk bounds (nc + 1) | 0 .. nc - 1 | nc zeros | nc ones | each
+// sequence's first chunk (nseq + 1)], built by the caller from the step's run lengths; absent: token by token.
 void hgrn2_scan(Tensor p, int64_t H, int64_t dk, int64_t dv, Tensor f_bias, Tensor lower, Tensor norm_w, double eps,
-                Tensor state, Tensor seq_start, Tensor seq_slot, Tensor seq_init, Tensor out) {
+                Tensor state, Tensor seq_start, Tensor seq_slot, Tensor seq_init, Tensor out,
+                std::optional<Tensor> chunks, int64_t nc) {
   const c10::hip::OptionalHIPGuard g(dev_of(p));
   TORCH_CHECK(H >= 1 && dk >= 1 && dv >= 1, "head count and sizes");
   TORCH_CHECK(p.is_cuda() && act_ok(p) && p.dim() == 2 && p.stride(1) == 1 && p.size(1) >= 2 * H * dk + H * dv,
@@ -786,12 +789,27 @@ void hgrn2_scan(Tensor p, int64_t H, int64_t dk, int64_t dv, Tensor f_bias, Tens
   TORCH_CHECK(seq_slot.numel() <= 65535, "too many sequences in a step");
   // fp32 workspaces of the three kernels: [qn | kn | dec | o_raw]
   const int64_t n_qk = T * H * KD, n_o = T * H * dv;
-  Tensor ws = torch::empty({3 * n_qk + n_o + 4}, torch::dtype(torch::kFloat32).device(p.device()));
+  const int64_t nseq = seq_slot.numel();
+  const int* ch = nullptr;
+  int64_t n_cs = 0, n_cd = 0;
+  if (chunks) {
+    CHECK_I32(*chunks);
+    TORCH_CHECK(nc >= 1 && nc <= 65535 && chunks->numel() == 4 * nc + 1 + nseq + 1, "chunk table");
+    ch = chunks->data_ptr<int>();
+    n_cs = nc * H * dk * dv;
+    n_cd = nc * H * KD;
+  } else {
+    nc = 0;
+  }
+  Tensor ws = torch::empty({3 * n_qk + n_o + n_cs + n_cd + 4}, torch::dtype(torch::kFloat32).device(p.device()));
   float* w0 = ws.data_ptr<float>();
+  float* wc = w0 + 3 * n_qk + n_o;
   const int rc = sm_hgrn2_scan(p.data_ptr(), p.stride(0), H, dk, dv, f_bias.data_ptr<float>(), lower.data_ptr<float>(),
                                norm_w.data_ptr(), (float)eps, state.data_ptr<float>(), seq_start.data_ptr<int>(),
                                seq_slot.data_ptr<int>(), seq_init.data_ptr<int>(), out.data_ptr(), w0, w0 + n_qk,
-                               w0 + 2 * n_qk, w0 + 3 * n_qk, T, seq_slot.numel(), is_f32(p), cur());
+                               w0 + 2 * n_qk, w0 + 3 * n_qk, T, nseq, is_f32(p), nc, ch, ch ? ch + nc + 1 : nullptr,
+                               ch ? ch + 2 * nc + 1 : nullptr, ch ? ch + 3 * nc + 1 : nullptr,
+                               ch ? ch + 4 * nc + 1 : nullptr, wc, wc + n_cs, cur());
   TORCH_CHECK(rc == 0, "hgrn2_scan: key size above 256");
 }
 

@@ -114,12 +114,13 @@ __device__ __forceinline__ float group_sum(float v) {
 // tokens from one buffer, the next block's loads are in flight into registers, and are written to the
 // other buffer afterwards - the recurrence never waits for global memory. Per token a lane reads its
 // KR rows of k, q (and g) as 16-byte LDS broadcasts.
-template <typename T, int KR, int RG, bool CH, int TB, bool DELTA = true>
+// OUT = false: the state alone is advanced (no read-out) - the first pass of the chunked form below.
+template <typename T, int KR, int RG, bool CH, int TB, bool DELTA = true, bool OUT = true>
 __global__ __launch_bounds__(64) void gated_delta_scan_kernel(
     const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ dec,
     const float* __restrict__ beta, const T* __restrict__ xc, int64_t x_stride, int voff, int G, int dk, int H, int dv,
     float* __restrict__ state, const int* __restrict__ seq_start, const int* __restrict__ seq_slot,
-    const int* __restrict__ seq_init, float* __restrict__ o_raw) {
+    const int* __restrict__ seq_init, float* __restrict__ o_raw, float* __restrict__ run_decay = nullptr) {
   constexpr int KD = RG * KR, CPW = 64 / RG, NV = CH ? 3 : 2;       // vectors per token: k, q (, g)
   constexpr int C4 = KD / 4;                         // 16-byte chunks per vector
   constexpr int NL = TB * NV * C4 / 64;              // chunks per lane and block (KD >= 32: a whole number)
@@ -138,6 +139,11 @@ __global__ __launch_bounds__(64) void gated_delta_scan_kernel(
   float S[KR];
 #pragma unroll
   for (int i = 0; i < KR; ++i) S[i] = (init && colok && row0 + i < dk) ? sp[(int64_t)(row0 + i) * dv + col] : 0.f;
+  // pass 1 of the chunked form: the waves of a head's first column block also multiply the run's decays
+  const bool want_decay = !OUT && CH && run_decay != nullptr && cb == 0;
+  float D[(!OUT && CH) ? KR : 1];
+#pragma unroll
+  for (int i = 0; i < ((!OUT && CH) ? KR : 1); ++i) D[i] = 1.f;
   // one token: kp, qp, gp point at this lane's KR rows of k, q and (CH) g; returns the read-out
   auto token = [&](const float4* kp, const float4* qp, const float4* gp, float gj, float bj, float vj) {
     float k[KR];
@@ -149,6 +155,9 @@ __global__ __launch_bounds__(64) void gated_delta_scan_kernel(
       if (CH) {
         const float4 g4 = gp[i >> 2];
         S[i] *= g4.x; S[i + 1] *= g4.y; S[i + 2] *= g4.z; S[i + 3] *= g4.w;
+        if (!OUT && want_decay) {
+          D[i] *= g4.x; D[i + 1] *= g4.y; D[i + 2] *= g4.z; D[i + 3] *= g4.w;
+        }
       } else {
         S[i] *= gj; S[i + 1] *= gj; S[i + 2] *= gj; S[i + 3] *= gj;
       }
@@ -166,12 +175,14 @@ __global__ __launch_bounds__(64) void gated_delta_scan_kernel(
     for (int i = 0; i < KR; i += 4) {
       const float4 q4 = qp[i >> 2];
       S[i] += k[i] * u; S[i + 1] += k[i + 1] * u; S[i + 2] += k[i + 2] * u; S[i + 3] += k[i + 3] * u;
-      o[0] += S[i] * q4.x;
-      o[1] += S[i + 1] * q4.y;
-      o[2] += S[i + 2] * q4.z;
-      o[3] += S[i + 3] * q4.w;
+      if (OUT) {
+        o[0] += S[i] * q4.x;
+        o[1] += S[i + 1] * q4.y;
+        o[2] += S[i + 2] * q4.z;
+        o[3] += S[i + 3] * q4.w;
+      }
     }
-    return group_sum<RG>((o[0] + o[1]) + (o[2] + o[3]));
+    return OUT ? group_sum<RG>((o[0] + o[1]) + (o[2] + o[3])) : 0.f;
   };
   if (hi - lo <= 2) {
     // a decoded token (or two): the lane's rows straight from global memory, no staging
@@ -181,7 +192,7 @@ __global__ __launch_bounds__(64) void gated_delta_scan_kernel(
       const float4* gp = reinterpret_cast<const float4*>(CH ? dec + (t * H + h) * KD + row0 : kn);
       const float vj = colok ? ld(xc + t * x_stride + voff + h * dv + col) : 0.f;
       const float ov = token(kp, qp, gp, CH ? 1.f : dec[t * H + h], DELTA ? beta[t * H + h] : 1.f, vj);
-      if (r == 0 && colok) o_raw[t * H * dv + h * dv + col] = ov;
+      if (OUT && r == 0 && colok) o_raw[t * H * dv + h * dv + col] = ov;
     }
   } else {
     float4 stage[NL];
@@ -238,7 +249,7 @@ __global__ __launch_bounds__(64) void gated_delta_scan_kernel(
                                reinterpret_cast<const float4*>(bk + (j * NV + 1) * KD + row0),
                                reinterpret_cast<const float4*>(bk + (j * NV + (CH ? 2 : 0)) * KD + row0),
                                CH ? 1.f : cg[j], cbeta[j], cv[j]);
-        if (r == 0 && colok) o_raw[(int64_t)(t0 + j) * H * dv + h * dv + col] = ov;
+        if (OUT && r == 0 && colok) o_raw[(int64_t)(t0 + j) * H * dv + h * dv + col] = ov;
       }
       if (more) spill(which ^ 1);
       __syncthreads();  // one wave: orders the buffer's writes before the next block's reads
@@ -248,6 +259,41 @@ __global__ __launch_bounds__(64) void gated_delta_scan_kernel(
 #pragma unroll
     for (int i = 0; i < KR; ++i)
       if (row0 + i < dk) sp[(int64_t)(row0 + i) * dv + col] = S[i];
+  }
+  if (!OUT && CH && want_decay && c == 0) {
+#pragma unroll
+    for (int i = 0; i < KR; ++i) run_decay[((int64_t)s * H + h) * KD + row0 + i] = D[i];
+  }
+}
+
+// Chunked form of the recurrence without the delta term, for prompts: S <- diag(g) S + k v^T is linear in
+// S, so a run cut into chunks can be scanned in all chunks at once. Pass 1 scans every chunk from zero
+// (its own contribution L_c, no read-out) and multiplies the chunk's decays (D_c, one per key row); the
+// small kernel below walks a sequence's chunks in order, S_(c+1) = D_c S_c + L_c, leaving every
+// chunk's true start state where its L_c was and the run's final state in the sequence's slot; pass 2
+// scans every chunk again from its start state and reads out. All fp32; against the token-by-token scan
+// only the order of the additions that form a chunk's start state differs.
+// c_state [chunks, H, dk, dv]: in L_c, out the start state of chunk c. s_chunk0 [nseq + 1] bounds each
+// sequence's chunks.
+__global__ __launch_bounds__(NT) void chunk_link_kernel(float* __restrict__ c_state, const float* __restrict__ c_decay,
+                                                       const int* __restrict__ s_chunk0, int H, int dk, int dv, int KD,
+                                                       float* __restrict__ state, const int* __restrict__ seq_slot,
+                                                       const int* __restrict__ seq_init) {
+  const int s = blockIdx.y;
+  const int64_t n = (int64_t)H * dk * dv;
+  const int c0 = s_chunk0[s], c1 = s_chunk0[s + 1];
+  if (c0 >= c1) return;
+  float* sp = state + (int64_t)seq_slot[s] * n;
+  const bool init = seq_init[s] != 0;
+  for (int64_t e = (int64_t)blockIdx.x * NT + threadIdx.x; e < n; e += (int64_t)gridDim.x * NT) {
+    const int h = (int)(e / ((int64_t)dk * dv)), i = (int)((e / dv) % dk);
+    float S = init ? sp[e] : 0.f;
+    for (int c = c0; c < c1; ++c) {
+      const float own = c_state[(int64_t)c * n + e];
+      c_state[(int64_t)c * n + e] = S;
+      S = c_decay[((int64_t)c * H + h) * KD + i] * S + own;
+    }
+    sp[e] = S;
   }
 }
 
@@ -331,38 +377,54 @@ int sm_gated_delta_scan(const void* xc, int64_t x_stride, int G, int dk, int H, 
 
 // HGRN2 over the projection p = [q | f | v] (H dk, H dk, H dv columns). Workspaces (fp32): qn, kn, dec
 // [T, H, KD]; o_raw [T, H, dv]. Returns 0, or 1 when the key size does not fit (dk > 256).
+// nc > 0: the chunked form. c_start [nc + 1] bounds the chunks (every run cut into pieces), c_slot = 0 .. nc - 1,
+// c_zero / c_one [nc] are all 0 / all 1, s_chunk0 [nseq + 1] bounds each sequence's chunks; c_state
+// [nc, H, dk, dv] and c_decay [nc, H, KD] are fp32 scratch.
 int sm_hgrn2_scan(const void* p, int64_t p_stride, int H, int dk, int dv, const float* f_bias, const float* lower,
                   const void* norm_w, float eps, float* state, const int* seq_start, const int* seq_slot,
                   const int* seq_init, void* out, float* qn, float* kn, float* dec, float* o_raw, int T, int nseq,
-                  int f32, hipStream_t stream) {
+                  int f32, int nc, const int* c_start, const int* c_slot, const int* c_zero, const int* c_one,
+                  const int* s_chunk0, float* c_state, float* c_decay, hipStream_t stream) {
   if (nseq == 0 || T == 0) return 0;
   const int KD = sm_gated_delta_rows(dk);
   if (KD == 0) return 1;
   const int voff = 2 * H * dk;
-  const bool wide = (int64_t)nseq * H * ((dv + 15) / 16) >= 1024;
+  const int nrun = nc > 0 ? nc : nseq;  // runs the scan kernel sees
+  const bool wide = (int64_t)nrun * H * ((dv + 15) / 16) >= 1024;
   const int cpw = wide ? 16 : 8;
-  const dim3 grid(H * ((dv + cpw - 1) / cpw), nseq);
+  const dim3 grid(H * ((dv + cpw - 1) / cpw), nrun);
   const dim3 pgrid(T, std::max(1, std::min((H * KD + NT - 1) / NT, 4096 / T)));
   const dim3 ogrid(T, std::max(1, std::min((H + 3) / 4, 4096 / T)));
-#define SM_GO(TYPE, KR, RG)                                                                                          \
-  hipLaunchKernelGGL((gated_delta_scan_kernel<TYPE, KR, RG, true, (KR * RG <= 128 ? 16 : 8), false>), grid, dim3(64), \
-                     0, stream, qn, kn, dec, nullptr, (const TYPE*)p, p_stride, voff, H, dk, H, dv, state, seq_start, \
-                     seq_slot, seq_init, o_raw)
-#define SM_RG(TYPE, KD_)              \
-  if (wide) SM_GO(TYPE, KD_ / 4, 4);  \
-  else SM_GO(TYPE, KD_ / 8, 8)
+#define SM_GO(TYPE, KR, RG, OUT_, ST, START, SLOT, INIT)                                                              \
+  hipLaunchKernelGGL((gated_delta_scan_kernel<TYPE, KR, RG, true, (KR * RG <= 128 ? 16 : 8), false, OUT_>), grid,      \
+                     dim3(64), 0, stream, qn, kn, dec, nullptr, (const TYPE*)p, p_stride, voff, H, dk, H, dv, ST,      \
+                     START, SLOT, INIT, o_raw, c_decay)
+#define SM_RG(TYPE, KD_, ...)                      \
+  if (wide) SM_GO(TYPE, KD_ / 4, 4, __VA_ARGS__);  \
+  else SM_GO(TYPE, KD_ / 8, 8, __VA_ARGS__)
+#define SM_KD(TYPE, ...)                                     \
+  if (KD == 32) { SM_RG(TYPE, 32, __VA_ARGS__); }            \
+  else if (KD == 64) { SM_RG(TYPE, 64, __VA_ARGS__); }       \
+  else if (KD == 128) { SM_RG(TYPE, 128, __VA_ARGS__); }     \
+  else { SM_RG(TYPE, 256, __VA_ARGS__); }
 #define SM_ALL(TYPE)                                                                                                 \
   hipLaunchKernelGGL((hgrn2_prep_kernel<TYPE>), pgrid, dim3(NT), 0, stream, (const TYPE*)p, p_stride, H, dk, KD,      \
                      f_bias, lower, qn, kn, dec);                                                                    \
-  if (KD == 32) { SM_RG(TYPE, 32); }                                                                                 \
-  else if (KD == 64) { SM_RG(TYPE, 64); }                                                                            \
-  else if (KD == 128) { SM_RG(TYPE, 128); }                                                                          \
-  else { SM_RG(TYPE, 256); }                                                                                         \
+  if (nc > 0) {                                                                                                      \
+    SM_KD(TYPE, false, c_state, c_start, c_slot, c_zero)                                                             \
+    hipLaunchKernelGGL(chunk_link_kernel, dim3((unsigned)std::min<int64_t>(((int64_t)H * dk * dv + NT - 1) / NT, 2048), \
+                                               nseq), dim3(NT), 0, stream, c_state, c_decay, s_chunk0, H, dk, dv, KD, \
+                       state, seq_slot, seq_init);                                                                   \
+    SM_KD(TYPE, true, c_state, c_start, c_slot, c_one)                                                               \
+  } else {                                                                                                           \
+    SM_KD(TYPE, true, state, seq_start, seq_slot, seq_init)                                                          \
+  }                                                                                                                  \
   hipLaunchKernelGGL((delta_out_kernel<TYPE>), ogrid, dim3(NT), 0, stream, o_raw, (const TYPE*)nullptr, (int64_t)0, 0, \
                      (const TYPE*)norm_w, eps, H, dv, (TYPE*)out)
   if (f32) { SM_ALL(float); }
   else { SM_ALL(bf16_t); }
 #undef SM_ALL
+#undef SM_KD
 #undef SM_RG
 #undef SM_GO
   return 0;

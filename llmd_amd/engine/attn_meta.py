@@ -30,6 +30,7 @@ class SeqMeta:
     q_lens: Optional[list] = None    # host copy of the run lengths
     ctx_lens: Optional[list] = None  # host copy of each sequence's context length after the step
     _items: Optional[dict] = None    # (tokens per item, balance) -> [n, 3] int32 work items (attention_items)
+    _chunks: Optional[dict] = None   # chunk length -> (table, number of chunks) (scan_chunks)
 
     def attention_items(self, tokens_per_item: int, balance: int = 0) -> torch.Tensor:
         """Work items (sequence, first token row, tokens) of the matrix-core attention kernel: every
@@ -65,6 +66,32 @@ class SeqMeta:
                 it = it.pin_memory().to(self.tables.device, non_blocking=True)
             self._items[key] = it
         return it
+
+
+    def _scan_chunks(self, length: int):
+        bounds, first = [0], [0]
+        for n in self.q_lens:
+            t0 = bounds[-1]
+            for a in range(0, n, length):
+                bounds.append(t0 + min(n, a + length))
+            first.append(len(bounds) - 1)
+        nc = len(bounds) - 1
+        table = torch.tensor(bounds + list(range(nc)) + [0] * nc + [1] * nc + first, dtype=torch.int32)
+        if self.tables.is_cuda:
+            table = table.pin_memory().to(self.tables.device, non_blocking=True)
+        return table, nc
+
+    def scan_chunks(self, length: int):
+        """Every run cut into chunks of at most ``length`` tokens, for recurrences that are linear in their
+        state and scan the chunks of a prompt side by side. Returns (table, nc): int32 [chunk bounds
+        (nc + 1) | 0 .. nc - 1 | nc zeros | nc ones | first chunk of each sequence (n + 1)] - the bounds,
+        scratch slots and "start from zero" / "continue" flags of the chunks as runs of their own, and each
+        sequence's range of chunks. Built once per step and length."""
+        if self._chunks is None:
+            self._chunks = {}
+        if length not in self._chunks:
+            self._chunks[length] = self._scan_chunks(length)
+        return self._chunks[length]
 
 
 @dataclass

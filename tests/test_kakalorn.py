@@ -275,6 +275,45 @@ def test_hgrn2_remembers_far_back_when_it_forgets_slowly(device, dtype):
     assert rel_err(got, want) < _tol(dtype, 2e-4, 3e-2)
 
 
+@pytest.mark.parametrize("device,dtype", ATT_DTYPES)
+@pytest.mark.parametrize("H,dk,dv", [(2, 16, 24), (3, 10, 70), (2, 130, 136), (1, 64, 64), (1, 1, 1)])
+def test_hgrn2_long_portions_are_scanned_in_chunks(device, dtype, H, dk, dv):
+    """Portions long enough for the chunked form (their chunks scanned side by side and linked), between
+    short ones and single tokens: chunk ends that fall on, before and after the portions' ends."""
+    for steps in ([700], [257, 1, 300, 2, 1024, 1], [3, 640, 1, 1, 256]):
+        got, want = _hgrn2_case(device, dtype, H, dk, dv, steps, seed=len(steps))
+        assert rel_err(got, want) < _tol(dtype, 2e-4, 3e-2)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_hgrn2_chunked_step_of_several_sequences(device):
+    """A long portion beside a short one, a single token and a second long one in the same step, each
+    continuing its own slot: the same rows as each sequence alone, token by token."""
+    H, dk, dv = 2, 16, 24
+    g = torch.Generator().manual_seed(5)
+    fb, low = torch.randn(H * dk, generator=g).to(device), torch.rand(H * dk, generator=g).to(device)
+    nw = torch.ones(dv, device=device)
+    lens = [(40, 300), (3, 5), (7, 1), (0, 513)]                  # (tokens in the first step, tokens in the second)
+    ps = [torch.randn(a + b, 2 * H * dk + H * dv, generator=g).to(device) for a, b in lens]
+    alone = []
+    for p in ps:
+        st = torch.zeros(1, H, dk, dv, device=device)
+        alone.append(torch.cat([sm.hgrn2_scan(p[t:t + 1], H, dk, dv, fb, low, nw, 1e-5, st, _seq(device, [1], [0], [int(t > 0)]))
+                                for t in range(p.shape[0])]))
+    state = torch.randn(5, H, dk, dv, generator=g).to(device)
+    slots = [3, 0, 4, 1]
+    first = [i for i, (a, _) in enumerate(lens) if a]
+    o1 = sm.hgrn2_scan(torch.cat([ps[i][:lens[i][0]] for i in first]), H, dk, dv, fb, low, nw, 1e-5, state,
+                       _seq(device, [lens[i][0] for i in first], [slots[i] for i in first], [0] * len(first)))
+    o2 = sm.hgrn2_scan(torch.cat([p[a:] for p, (a, _) in zip(ps, lens)]), H, dk, dv, fb, low, nw, 1e-5, state,
+                       _seq(device, [b for _, b in lens], slots, [int(a > 0) for a, _ in lens]))
+    t1 = t2 = 0
+    for i, (a, b) in enumerate(lens):
+        got = torch.cat([o1[t1:t1 + a], o2[t2:t2 + b]])
+        t1, t2 = t1 + a, t2 + b
+        assert rel_err(got, alone[i].double().cpu()) < 2e-5, i
+
+
 @pytest.mark.parametrize("device", DEVICES)
 def test_hgrn2_state_slots_are_separate(device):
     """Two sequences in one step continue their own slots; a new sequence in a used slot starts from zero."""
