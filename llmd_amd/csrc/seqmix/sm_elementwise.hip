@@ -192,6 +192,99 @@ __global__ __launch_bounds__(NT) void post_norm_add_kernel(const T* __restrict__
   for (int c = threadIdx.x; c < d; c += NT) st(out + row * d + c, xr[c] * inv2 * ld(wn + c));
 }
 
+// The same for bf16 rows of d = 8 n <= 8 * NT * NCH elements with 16-byte accesses: a thread keeps its
+// NCH chunks of eight elements in registers from the first pass to the last, so y is read once, x read
+// and written once and out written once; a small step's rows are a few loads deep instead of d / NT.
+template <int NCH>
+__global__ __launch_bounds__(NT) void post_norm_add_vec_kernel(const bf16_t* __restrict__ y, int64_t y_stride,
+                                                              const bf16_t* __restrict__ y2, int64_t y2_stride,
+                                                              float a, float b, const float* __restrict__ bias,
+                                                              const bf16_t* __restrict__ wp, float* __restrict__ x,
+                                                              float eps, const bf16_t* __restrict__ wn,
+                                                              bf16_t* __restrict__ out, int d) {
+  __shared__ float red[NT / 64];
+  const int64_t row = blockIdx.x;
+  auto ld8 = [](const bf16_t* p, float* v) {
+    const uint4 q = *reinterpret_cast<const uint4*>(p);
+    v[0] = __uint_as_float(q.x << 16); v[1] = __uint_as_float(q.x & 0xffff0000u);
+    v[2] = __uint_as_float(q.y << 16); v[3] = __uint_as_float(q.y & 0xffff0000u);
+    v[4] = __uint_as_float(q.z << 16); v[5] = __uint_as_float(q.z & 0xffff0000u);
+    v[6] = __uint_as_float(q.w << 16); v[7] = __uint_as_float(q.w & 0xffff0000u);
+  };
+  auto ldf8 = [](const float* p, float* v) {
+    const float4 q0 = *reinterpret_cast<const float4*>(p), q1 = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = q0.x; v[1] = q0.y; v[2] = q0.z; v[3] = q0.w; v[4] = q1.x; v[5] = q1.y; v[6] = q1.z; v[7] = q1.w;
+  };
+  auto pack = [](float lo_, float hi_) {
+    const __bf16 l16 = (__bf16)lo_, h16 = (__bf16)hi_;
+    return (uint32_t)__builtin_bit_cast(uint16_t, l16) | ((uint32_t)__builtin_bit_cast(uint16_t, h16) << 16);
+  };
+  float v[NCH][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < NCH; ++k) {
+    const int c = (k * NT + threadIdx.x) * 8;
+    if (c < d) {
+      ld8(y + row * y_stride + c, v[k]);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[k][i] *= a;
+      if (y2) {
+        float t[8];
+        ld8(y2 + row * y2_stride + c, t);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[k][i] += b * t[i];
+      }
+      if (bias) {
+        float t[8];
+        ldf8(bias + c, t);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[k][i] += t[i];
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) ss += v[k][i] * v[k][i];
+    }
+  }
+  ss = block_sum<NT>(ss, red);
+  const float inv = 1.f / sqrtf(ss / (float)d + eps);
+  float s2 = 0.f;
+#pragma unroll
+  for (int k = 0; k < NCH; ++k) {
+    const int c = (k * NT + threadIdx.x) * 8;
+    if (c < d) {
+      float xv[8], w[8];
+      ldf8(x + row * d + c, xv);
+      ld8(wp + c, w);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        v[k][i] = xv[i] + v[k][i] * inv * w[i];
+        s2 += v[k][i] * v[k][i];
+      }
+      float* xr = x + row * d + c;
+      *reinterpret_cast<float4*>(xr) = make_float4(v[k][0], v[k][1], v[k][2], v[k][3]);
+      *reinterpret_cast<float4*>(xr + 4) = make_float4(v[k][4], v[k][5], v[k][6], v[k][7]);
+    }
+  }
+  float inv2 = 1.f;
+  if (wn != nullptr) {
+    s2 = block_sum<NT>(s2, red);
+    inv2 = 1.f / sqrtf(s2 / (float)d + eps);
+  }
+#pragma unroll
+  for (int k = 0; k < NCH; ++k) {
+    const int c = (k * NT + threadIdx.x) * 8;
+    if (c < d) {
+      float w[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};
+      if (wn != nullptr) ld8(wn + c, w);
+      uint4 o;
+      o.x = pack(v[k][0] * inv2 * w[0], v[k][1] * inv2 * w[1]);
+      o.y = pack(v[k][2] * inv2 * w[2], v[k][3] * inv2 * w[3]);
+      o.z = pack(v[k][4] * inv2 * w[4], v[k][5] * inv2 * w[5]);
+      o.w = pack(v[k][6] * inv2 * w[6], v[k][7] * inv2 * w[7]);
+      *reinterpret_cast<uint4*>(out + row * d + c) = o;
+    }
+  }
+}
+
 // x = table[id] (fp32 residual);  out = x / rms(x) * w
 template <typename T>
 __global__ __launch_bounds__(NT) void embed_norm_kernel(const int64_t* __restrict__ ids, const T* __restrict__ table,
@@ -343,6 +436,21 @@ void sm_post_norm_add(const void* y, int64_t y_stride, const void* y2, int64_t y
                       const float* bias, const void* wp, float* x, float eps, const void* wn, void* out, int T, int d,
                       int f32, hipStream_t stream) {
   if (T == 0) return;
+  const int nch = (d / 8 + NT - 1) / NT;
+  const bool aligned = (((uintptr_t)y | (uintptr_t)y2 | (uintptr_t)bias | (uintptr_t)wp | (uintptr_t)x | (uintptr_t)wn |
+                         (uintptr_t)out) & 15) == 0 && y_stride % 8 == 0 && y2_stride % 8 == 0;
+  if (!f32 && d % 8 == 0 && nch <= 4 && aligned) {
+#define SM_PNA(N)                                                                                                     \
+  hipLaunchKernelGGL(post_norm_add_vec_kernel<N>, dim3(T), dim3(NT), 0, stream, (const bf16_t*)y, y_stride,           \
+                     (const bf16_t*)y2, y2_stride, a, b, bias, (const bf16_t*)wp, x, eps, (const bf16_t*)wn,          \
+                     (bf16_t*)out, d)
+    if (nch <= 1) SM_PNA(1);
+    else if (nch == 2) SM_PNA(2);
+    else if (nch == 3) SM_PNA(3);
+    else SM_PNA(4);
+#undef SM_PNA
+    return;
+  }
   if (f32)
     hipLaunchKernelGGL((post_norm_add_kernel<float>), dim3(T), dim3(NT), 0, stream, (const float*)y, y_stride,
                        (const float*)y2, y2_stride, a, b, bias, (const float*)wp, x, eps, (const float*)wn,

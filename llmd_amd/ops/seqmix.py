@@ -270,6 +270,10 @@ def qkv_rope_cache(qkv, bias, positions, cos_sin, Hq, Hkv, dim, vdim, rot_dims, 
 
 GQA_MFMA = os.environ.get("LLMD_GQA_MFMA", "1") == "1"
 GQA_DECODE_WGS = int(os.environ.get("LLMD_GQA_DECODE_WGS", "2048"))  # workgroups a decode-only step aims for
+# ... and with a sliding window: a row's keys are few, so a range's fixed work (query fragments, partial
+# results, the merge) weighs more. 64 sequences x 8 kv heads, window 1024 at context 2048, ms per layer of
+# the whole stack: 0.225 / 0.247 / 0.263 / 0.287 for 512 / 1024 / 2048 / 4096
+GQA_WINDOW_DECODE_WGS = int(os.environ.get("LLMD_GQA_WINDOW_DECODE_WGS", "512"))
 # LLMD_GQA_RB2=1: prompt portions run as 128-row items, two blocks of 16 rows per wave. Measured slower
 # than 64-row items at 128/128 heads (2048-token prompt: 227 us against 181 us - 185 + 64 registers
 # leave two waves per SIMD instead of three), so it stays an option.
@@ -317,7 +321,7 @@ def grouped_attention(q, cache, dim, vdim, scale: float, seq, gate=None, slopes=
             # decode-only step: key ranges so that items x kv heads x ranges give the chip about
             # eight workgroups per CU (a workgroup walks its tiles one after another)
             n = items.shape[0] * Hkv
-            nsplit = max(1, min(-(-GQA_DECODE_WGS // n), span // 128))
+            nsplit = max(1, min(-(-(GQA_WINDOW_DECODE_WGS if window else GQA_DECODE_WGS) // n), span // 128))
             split = -(-span // (nsplit * 32)) * 32
             nsplit = -(-span // split)
             if nsplit > 1:

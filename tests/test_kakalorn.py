@@ -186,7 +186,26 @@ def test_embedding_with_the_first_norm(device, dtype, d):
 
 
 @pytest.mark.parametrize("device,dtype", ATT_DTYPES)
-@pytest.mark.parametrize("n", [1, 12, 80, 333])
+@pytest.mark.parametrize("d", [40, 33, 2048, 4104, 8192, 8200])
+def test_norm_after_and_before_a_sublayer(device, dtype, d):
+    """x += norm(y) and, from the same pass, the next reader's norm of the new x (or x itself); rows that
+    are whole 16-byte pieces, rows that are not, and rows too long for a thread's registers."""
+    g = torch.Generator().manual_seed(d)
+    T = 5
+    y = torch.randn(T, d, generator=g).to(dtype)
+    w, wn = ((1 + 0.2 * torch.randn(d, generator=g)).to(dtype) for _ in range(2))
+    x0 = torch.randn(T, d, generator=g)
+    want_x = x0.double() + oracle.rms_norm(y.double(), w.double(), 1e-5)
+    for nxt in (wn, None):
+        x = x0.clone().to(device)
+        h = sm.post_norm_add(y.to(device), w.to(device), x, 1e-5, dtype, nxt.to(device) if nxt is not None else None)
+        want_h = want_x if nxt is None else oracle.rms_norm(want_x, nxt.double(), 1e-5)
+        assert rel_err(x, want_x) < 1e-5
+        assert h.dtype == dtype and rel_err(h.float(), want_h) < _tol(dtype)
+
+
+@pytest.mark.parametrize("device,dtype", ATT_DTYPES)
+@pytest.mark.parametrize("n", [1, 12, 80, 333, 1536])
 def test_row_norm_of_a_column_view(device, dtype, n):
     g = torch.Generator().manual_seed(n)
     p = torch.randn(11, n + 9, generator=g).to(dtype)
