@@ -354,7 +354,7 @@ def test_hgrn2_state_slots_are_separate(device):
     assert rel_err(again, alone[1].double().cpu()) < 1e-5
 
 
-@pytest.mark.parametrize("dims,base,scaling", [(8, 10000.0, None), (32, 500000.0, (2.0, 1024, 32.0, 1.0)),
+@pytest.mark.parametrize("dims,base,scaling", [(8, 10000.0, None), (32, 500000.0, (4.0, 2048, 16.0, 2.0)),
                                                (16, 100.0, (8.0, 4096, 1.0, 1.0)), (10, 777.0, (3.0, 40, 5.0, 0.5)),
                                                (64, 10000.0, (40.0, 4096, 32.0, 1.0))])
 def test_ramp_scaled_frequencies(dims, base, scaling):
@@ -451,7 +451,7 @@ def test_learned_sinks_show(device, dtype):
 @pytest.mark.parametrize("device,dtype", ATT_DTYPES)
 @pytest.mark.parametrize("Hq,Hkv,dim,rot,size,keep", [(6, 3, 24, 16, 20, 3), (5, 5, 10, 6, 64, 0), (8, 1, 64, 64, 300, 33),
                                                       (2, 2, 130, 128, 7, 70), (4, 2, 64, 32, 96, 1), (3, 1, 16, 0, 1, 0),
-                                                      (4, 4, 32, 32, 0, 0), (4, 1, 96, 96, 100, 12)])
+                                                      (4, 4, 32, 32, 0, 0), (6, 2, 96, 96, 100, 12)])
 @pytest.mark.parametrize("decode_only", [False, True], ids=["mixed-step", "decode-step"])
 def test_windowed_attention_steps(device, dtype, Hq, Hkv, dim, rot, size, keep, decode_only):
     """Several sequences of unequal length in one step, pages shuffled: single decoded tokens (one far
@@ -511,7 +511,7 @@ def test_windowed_attention_steps(device, dtype, Hq, Hkv, dim, rot, size, keep, 
 
 
 @pytest.mark.parametrize("device,dtype", ATT_DTYPES)
-@pytest.mark.parametrize("H,dn,dr,R,rot_dims", [(3, 16, 8, 20, 8), (6, 64, 32, 64, 32), (1, 8, 6, 5, 4), (5, 24, 16, 40, 16)])
+@pytest.mark.parametrize("H,dn,dr,R,rot_dims", [(3, 16, 8, 20, 8), (4, 64, 32, 96, 32), (1, 8, 6, 5, 4), (5, 24, 16, 40, 16)])
 def test_latent_rotation_pairs_and_cache_write(device, dtype, H, dn, dr, R, rot_dims):
     """Interleaved pairs with ramp-scaled angles on queries and on the shared key part; a layer without
     a down-projection of its own rotates its queries and leaves the cache alone."""
@@ -548,7 +548,7 @@ def test_latent_rotation_pairs_and_cache_write(device, dtype, H, dn, dr, R, rot_
 
 
 @pytest.mark.parametrize("device,dtype", ATT_DTYPES)
-@pytest.mark.parametrize("H,R,dr", [(3, 20, 8), (6, 64, 32), (1, 5, 6), (16, 128, 16)])
+@pytest.mark.parametrize("H,R,dr", [(3, 20, 8), (4, 96, 32), (1, 5, 6), (16, 128, 16)])
 @pytest.mark.parametrize("decode_only", [False, True], ids=["mixed-step", "decode-step"])
 def test_latent_attention_head_gates(device, dtype, H, R, dr, decode_only):
     """One sigmoid gate per (token, head), read as a column view of a wider projection; decoded rows far
