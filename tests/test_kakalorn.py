@@ -223,7 +223,7 @@ def test_squared_relu(device, dtype, shape):
 
 
 @pytest.mark.parametrize("device,dtype", ATT_DTYPES)
-@pytest.mark.parametrize("taps", [1, 2, 4, 7])
+@pytest.mark.parametrize("taps", [1, 2, 4, 7, 9])
 @pytest.mark.parametrize("C", [40, 300, 4104])
 def test_input_convolution_continues_each_sequence(device, dtype, taps, C):
     """Two sequences in portions over several steps (one token, two tokens, fewer tokens than taps, a
