@@ -128,7 +128,8 @@ def build_ops(jobs: int = 8, verbose: bool = False, debug: bool = False) -> Path
 def build_seqmix(jobs: int = 8, verbose: bool = False) -> Path:
     """Build ``llmd_amd/_C_seqmix``: the kernels of per-layer stacks (latent attention of any
     size, selective scan, delta rules, zero-centred and post norms, ungated and gated experts, hyper-connected
-    streams, grouped attention with separate key and value sizes; ``csrc/seqmix``). It is a
+    streams, grouped attention with separate key and value sizes, windows and sinks, HGRN2, input
+    convolutions; ``csrc/seqmix``). It is a
     library of its own so that a model that needs only these compiles only these."""
     tinc, tlib = _torch_paths()
     name = "_C_seqmix"

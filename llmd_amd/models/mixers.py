@@ -171,7 +171,7 @@ class LatentAttention(torch.nn.Module):
         sm.latent_rope_cache(q, kv, self.dkv_norm if kv is not None else None, self.eps, meta.positions, self.cos_sin,
                              H, dn, dr, self.rot_dims, R, meta.slot_mapping, cache, q_abs, self.interleaved)
         # absorb W_uk into the query: scores against the latent itself
-        qn = q.view(T, H, dn + dr)[:, :, :dn].transpose(0, 1)                       # [H, T, dn]
+        qn = q.reshape(T, H, dn + dr)[:, :, :dn].transpose(0, 1)                      # [H, T, dn]
         q_abs[:, :, :R].copy_(torch.bmm(qn, self.uk.view(H, dn, R)).transpose(0, 1))
         o_lat = sm.latent_attention(q_abs, cache, s.tables, s.row_seq, s.row_len, self.scale, R,
                                     rows_per_group=4 if s.max_q > 1 else 1, seq=s, gate=gate)
