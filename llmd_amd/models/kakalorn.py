@@ -9,7 +9,7 @@ Mixers (models/mixers.py):
   ``attention``         grouped attention whose values are the projected keys (no value projection),
                         biased q / k, weighted query / key norms ahead of a partial half-split rotation,
                         a sliding window that keeps the sequence's first tokens, a learned sink per head
-  ``hgrn2``             gated linear recurrence: the forget gate, bounded below, also sets what is written
+  ``hgrn2``             gated linear recurrence: forget gate f bounded below, write strength 1 - f
   ``latent_attention``  queries through a normed latent, interleaved rotary pairs with ramp-scaled
                         frequencies, one sigmoid gate per head; a layer with ``kv_from`` reads the latent
                         cache of an earlier layer with its own up-projections

@@ -24,7 +24,7 @@ constant is an argument, so another stack can reuse them.
   norms ahead of the rotation, a sliding window that keeps the sequence's first tokens, learned sinks.
 * ``LatentAttention`` options: queries through a normed latent of their own, interleaved rotary pairs,
   ramp-scaled frequencies, one sigmoid gate per head, the cache of an earlier layer instead of its own.
-* ``Hgrn2Mixer``       - gated linear recurrence whose forget gate (bounded below) also sets what is written.
+* ``Hgrn2Mixer``       - gated linear recurrence: forget gate f (bounded below), write strength 1 - f.
 * ``SquaredReluMLP``   - W_down relu(W_up h)^2.
 * ``InputConv``        - h + a short causal convolution of h, in front of a mixer.
 
@@ -598,7 +598,7 @@ class BigramEmbedding(torch.nn.Module):
 
 
 class Hgrn2Mixer(torch.nn.Module):
-    """Gated linear recurrence per head whose forget gate also decides what is written. One
+    """Gated linear recurrence per head: a row of the state that forgets with f is written with 1 - f. One
     projection of the layer input gives [q | f | v]: q = silu(.) [heads, dim], v [heads, vdim] and the
     gate f = lower + (1 - lower) sigmoid(. + f_bias) per head and channel, ``lower`` its bound from
     below. Per head, in fp32:
